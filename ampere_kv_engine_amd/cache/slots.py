@@ -3,7 +3,8 @@ does not grow with the sequence keeps it at `state[slot]`.  Slots are handed out
 freed slot is the next one taken.
 
 `SlotArrays` is what every request keeps on the device between steps whatever its mixers are: `SLOT_WORDS` 32-bit
-words (tokens held, the token chosen last, temperature, seed, draws made so far, whether the slot is taken) and one
+words (tokens held, the token chosen last, temperature, seed, draws made so far, whether the slot is taken, the
+token fed last) and one
 row of each cache group's block table.  The reference keeps all of this in Python objects and uploads the tables once
 per layer and step (ampere_kv/scheduler.py:14-34, ampere_kv/runner.py:207-213); here a step uploads only what changed -
 the table entries of pages that were handed out or given back - and the sampler reads and advances a request's
@@ -16,7 +17,7 @@ import struct
 import torch
 
 SLOT_WORDS = 8
-WORD_LENGTH, WORD_LAST_TOKEN, WORD_TEMPERATURE, WORD_SEED_LOW, WORD_SEED_HIGH, WORD_DRAWS, WORD_TAKEN = range(7)
+WORD_LENGTH, WORD_LAST_TOKEN, WORD_TEMPERATURE, WORD_SEED_LOW, WORD_SEED_HIGH, WORD_DRAWS, WORD_TAKEN, WORD_FED_TOKEN = range(8)
 NO_TOKEN = -1
 
 
@@ -46,7 +47,7 @@ class SlotArrays:
         bits = struct.unpack("<i", struct.pack("<f", float(temperature)))[0]
         low, high = seed & 0xFFFFFFFF, (seed >> 32) & 0xFFFFFFFF
         signed = lambda word: word - (1 << 32) if word >= (1 << 31) else word
-        fresh = torch.tensor([0, NO_TOKEN, bits, signed(low), signed(high), 0, 1, 0], dtype=torch.int32)
+        fresh = torch.tensor([0, NO_TOKEN, bits, signed(low), signed(high), 0, 1, NO_TOKEN], dtype=torch.int32)
         if self.device.type == "cuda":
             # pinned memory from torch's caching host allocator, which keeps it until the copy has been made
             self.words[slot].copy_(fresh.pin_memory(), non_blocking=True)

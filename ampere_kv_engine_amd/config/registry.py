@@ -1,4 +1,5 @@
-"""The one registry from an architecture's name (config.json `architectures[0]`) to its typed configuration.
+"""The one registry from an architecture's name (config.json `architectures[0]`, or the one name under `architecture`)
+to its typed configuration.
 
 An entry is a configuration class with `from_folder(folder)` and `to_model_spec()`.  The model itself is
 always assembled from the `ModelSpec` by the part registries, so registering an architecture means
@@ -11,6 +12,7 @@ import json
 import os
 from typing import Protocol
 
+from .keranex import KeranexConfig
 from .qwen3 import ConfigError, Qwen3Config
 from .specs import ModelSpec
 
@@ -44,6 +46,8 @@ def architecture_of(folder: str) -> str:
     with open(path) as handle:
         raw = json.load(handle)
     names = raw.get("architectures")
+    if names is None and isinstance(raw.get("architecture"), str):      # the key some designs write: one name, no list
+        names = [raw["architecture"]]
     if not isinstance(names, list) or len(names) != 1 or not isinstance(names[0], str):
         raise ConfigError(f"config.json key architectures must be a list with one name, got {names!r}")
     return names[0]
@@ -58,3 +62,4 @@ def load_config(folder: str) -> ArchitectureConfig:
 
 
 register_architecture(Qwen3Config.architecture, Qwen3Config)
+register_architecture(KeranexConfig.architecture, KeranexConfig)

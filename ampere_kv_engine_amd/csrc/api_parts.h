@@ -1,0 +1,68 @@
+// C entry points of the second kernel library (`libakv_parts.so`): the token-wise kernels, mixers and routed
+// feed-forward of designs that keep their residual sum and norms in float32 throughout.  Conventions as in api.h:
+// every function enqueues on `stream` and returns 0, a hipError_t of the launch, -1 for an unknown dtype code or -2 for
+// sizes the kernel does not take.  dtype codes: 0 float32, 1 bfloat16.  Shapes are checked by the caller on the host.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+extern "C" {
+
+// ---- token-wise (tokenwise_f32.hip) ---------------------------------------------------------------------------------
+// out[n] = table[id] + pairs[row], row = (previous id * mul_prev + id * mul_cur) mod buckets, or `buckets` for a
+// request's first token.  The previous id of a portion's first token is the word `fed` of the request's slot.
+int akv_embed_pairs(const int* ids, const void* table, const void* pairs, int dtype, float* out, int tokens, int hidden,
+                    int vocab, long buckets, long mul_prev, long mul_cur, const int* seq_of_token, const int* q_start,
+                    const int* positions, const int* seq_slots, int* slot_words, hipStream_t stream);
+// word `fed` of every request's slot = the id of the last token it brought in this step
+int akv_note_fed_tokens(const int* ids, const int* q_start, const int* seq_slots, int* slot_words, int seqs,
+                        hipStream_t stream);
+// stream [tokens, hidden] float32.  With `delta` (dtype): stream += delta / rms(delta) * post_weight (or += delta where
+// post_weight is null).  With `out` (dtype): out = stream / rms(stream) * pre_weight, rounded once.
+int akv_norm_add_norm(float* stream_buf, const void* delta, const float* post_weight, float post_eps,
+                      const float* pre_weight, float pre_eps, void* out, int dtype, int tokens, int hidden,
+                      hipStream_t stream);
+
+// ---- attention over a compressed latent (latent_attention.hip) ------------------------------------------------------
+// down [tokens, q_rank (+ kv_rank + rot)]: q latent normed into `cq`; with `records`: the kv latent normed and the
+// shared key part rotated (first `rot_dims` of its `rot` dimensions) into the token's record [kv_rank + rot].
+int akv_latent_encode(const void* down, int dtype, int tokens, int q_rank, int kv_rank, int rot, int rot_dims,
+                      const float* q_weight, const float* kv_weight, float eps, const float* table, int table_positions,
+                      const int* positions, const int* slot_map, void* cq, void* records, long record_slots,
+                      hipStream_t stream);
+// q [tokens, heads, dim + rot] -> q_abs[..., at : at + rot] (float32, row width `width`), rotated by position
+int akv_rotate_queries(const void* q, int dtype, long tokens, int heads, int dim, int rot, int rot_dims,
+                       const float* table, int table_positions, const int* positions, float* q_abs, int width, int at,
+                       hipStream_t stream);
+// y[t, h, j] = sum_i x[t, h, i] * w[h, i, j]   (w [heads, ins, outs]; x and y addressed by token and head strides)
+int akv_heads_linear(const void* x, int x_dtype, long x_token_stride, long x_head_stride, const void* w, int w_dtype,
+                     void* y, int y_dtype, long y_token_stride, long y_head_stride, int tokens, int heads, int ins,
+                     int outs, hipStream_t stream);
+// out[t, h, :kv_rank] = softmax over the window of (q_abs[t, h] . record) * scale, times the records' first kv_rank
+int akv_latent_attend(const float* q_abs, const void* records, int dtype, const int* seq_of_token, const int* positions,
+                      const int* block_table, const int* table_rows, int table_width, float* out, int tokens, int heads,
+                      int kv_rank, int width, int page_size, long num_pages, float scale, int window,
+                      hipStream_t stream);
+
+// ---- selective scan (selective_scan.hip) ----------------------------------------------------------------------------
+// x [tokens, channels] at `x_stride` per token; state [slots, state_stride] float32 holds (taps - 1) x channels at
+// `conv_at`.  out = silu(conv + bias).
+int akv_conv_silu(const void* x, long x_stride, int dtype, const void* weight, const void* bias, int w_dtype,
+                  const float* state, long state_stride, long conv_at, const int* seq_of_token, const int* q_start,
+                  const int* seq_slots, void* out, int tokens, int channels, int taps, hipStream_t stream);
+int akv_conv_state_update(const void* x, long x_stride, int dtype, float* state, long state_stride, long conv_at,
+                          const int* q_start, const int* seq_slots, int seqs, int channels, int taps,
+                          hipStream_t stream);
+// S [channels, n_state] at the start of a slot's state; dt (before softplus), bc = [B | C] float32
+int akv_selective_scan(const void* x, int dtype, const float* dt, const float* bc, const void* z, long z_stride,
+                       const float* a, const float* d, float* state, long state_stride, const int* q_start,
+                       const int* seq_slots, void* out, int seqs, int channels, int n_state, hipStream_t stream);
+
+// ---- routed feed-forward (routed.hip) -------------------------------------------------------------------------------
+// gates [tokens, experts] float32: the softmax score of the chosen experts, 0 elsewhere
+int akv_route(const void* x, int dtype, const float* router, float* gates, int tokens, int hidden, int experts,
+              int top, int groups, int keep, hipStream_t stream);
+// act[t, e * ff + j] = gates[t, e] * relu(up[t, e * ff + j])^2
+int akv_gate_relu_squared(const void* up, const float* gates, void* act, int dtype, long tokens, int experts, int ff,
+                          hipStream_t stream);
+}

@@ -22,6 +22,11 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 SOURCES = ("elementwise.hip", "gemm.hip", "gemm_mfma.hip", "gemm_mid.hip", "gemm_decode.hip", "attention.hip", "sampling.hip")
 HEADERS = ("common.h", "mfma_tiles.h", "api.h")
 LIBRARY = "libakv_kernels.so"
+# a second library, compiled when a model first needs it: token-wise kernels, mixers and the routed feed-forward of
+# designs whose norms and residual sum are float32 throughout
+PARTS_SOURCES = ("tokenwise_f32.hip", "latent_attention.hip", "selective_scan.hip", "routed.hip")
+PARTS_HEADERS = ("common.h", "api_parts.h")
+PARTS_LIBRARY = "libakv_parts.so"
 ATTENTION_SOURCE = "attention_mfma.hip"        # compiled once per head size, into its own small library
 DEFAULT_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 128, 192, 256)
 ARCH = "gfx950"
@@ -38,9 +43,9 @@ def _hipcc() -> str:
                        "built, and the engine has no other way to compute")
 
 
-def source_stamp(sources=None) -> str:
+def source_stamp(sources=None, headers=HEADERS) -> str:
     digest = hashlib.sha256()
-    for name in (SOURCES if sources is None else tuple(sources)) + HEADERS:
+    for name in (SOURCES if sources is None else tuple(sources)) + tuple(headers):
         with open(os.path.join(HERE, name), "rb") as handle:
             digest.update(name.encode() + b"\0" + handle.read())
     digest.update(" ".join(FLAGS).encode())
@@ -126,6 +131,56 @@ def ensure_built(verbose: bool = True) -> str:
     return library_path() or build(verbose)
 
 
+# ---- the second library -------------------------------------------------------------------------------------------
+
+def parts_library_path() -> str | None:
+    stamp = source_stamp(PARTS_SOURCES, PARTS_HEADERS)
+    for folder in (os.path.join(HERE, "_build"),
+                   os.path.join(tempfile.gettempdir(), f"akv_build_{os.getuid()}_{source_stamp()[:12]}")):
+        lib, mark = os.path.join(folder, PARTS_LIBRARY), os.path.join(folder, "stamp_parts")
+        if os.path.exists(lib) and os.path.exists(mark):
+            with open(mark) as handle:
+                if handle.read().strip() == stamp:
+                    return lib
+    return None
+
+
+def build_parts(verbose: bool = True) -> str:
+    hipcc = _hipcc()
+    out_dir = _build_dir()
+    started = time.time()
+    if verbose:
+        _log(f"compiling {len(PARTS_SOURCES)} HIP sources for {ARCH} into {out_dir}")
+
+    def compile_one(name: str) -> str:
+        obj = os.path.join(out_dir, name.replace(".hip", ".o"))
+        result = subprocess.run([hipcc, *FLAGS, "-c", os.path.join(HERE, name), "-o", obj], capture_output=True, text=True)
+        if result.returncode != 0:
+            raise RuntimeError(f"hipcc failed on {name}:\n{result.stderr}")
+        if verbose:
+            _log(f"compiled {name} ({time.time() - started:.0f} s)")
+        return obj
+
+    with ThreadPoolExecutor(max_workers=min(4, len(PARTS_SOURCES))) as pool:
+        objects = list(pool.map(compile_one, PARTS_SOURCES))
+    lib = os.path.join(out_dir, PARTS_LIBRARY)
+    partial = lib + f".{os.getpid()}.tmp"
+    result = subprocess.run([hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", *objects, "-o", partial],
+                            capture_output=True, text=True)
+    if result.returncode != 0:
+        raise RuntimeError(f"linking {PARTS_LIBRARY} failed:\n{result.stderr}")
+    os.replace(partial, lib)
+    with open(os.path.join(out_dir, "stamp_parts"), "w") as handle:
+        handle.write(source_stamp(PARTS_SOURCES, PARTS_HEADERS))
+    if verbose:
+        _log(f"linked {lib} ({time.time() - started:.0f} s)")
+    return lib
+
+
+def ensure_parts(verbose: bool = True) -> str:
+    return parts_library_path() or build_parts(verbose)
+
+
 # ---- the attention kernels, one library per head size ------------------------------------------------------------
 
 def _attention_names(head_dim: int) -> tuple[str, str]:
@@ -174,7 +229,7 @@ def ensure_attention(head_dim: int, verbose: bool = True) -> str:
 
 def build_all(head_dims=DEFAULT_HEAD_DIMS, verbose: bool = True) -> list[str]:
     """The kernel library and the attention libraries of the usual head sizes."""
-    paths = [build(verbose)]
+    paths = [build(verbose), build_parts(verbose)]
     with ThreadPoolExecutor(max_workers=4) as pool:
         paths += list(pool.map(lambda d: build_attention(d, verbose), head_dims))
     return paths

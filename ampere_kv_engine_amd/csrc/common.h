@@ -74,6 +74,7 @@ enum SlotWord : int {
   kSlotSeedHigh = 4,
   kSlotDraws = 5,        // draws made so far
   kSlotTaken = 6,        // whether a request holds the slot
+  kSlotFedToken = 7,     // the token the request was fed last (what a model that looks at token pairs needs; -1: none)
 };
 
 // Blocks of one launch that hand sums to each other through memory do it in three steps.  (1) The sums are written

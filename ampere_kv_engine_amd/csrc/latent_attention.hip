@@ -1,0 +1,349 @@
+// Attention over a compressed latent, with a sliding window.
+//
+// A token's cache record is [c | k_rot]: the normed latent (kv_rank) and one rotated key part (rot) that all heads
+// share.  Keys and values of a head are linear in c (k_h = U_h c, v_h = V_h c), so the scores and the weighted sum can
+// be taken over the records themselves:
+//     q_h . k_h(j) = (U_h^T q_h) . c_j            sum_j p_j v_h(j) = V_h (sum_j p_j c_j)
+// `heads_linear` forms U_h^T q_h before and V_h (...) after; in between every head attends the same records - one
+// kv head whose keys are kv_rank + rot wide and whose values are the keys' first kv_rank dimensions.  Norms, angles,
+// scores, softmax and the weighted sums are float32.
+
+#include "common.h"
+#include "api_parts.h"
+
+using namespace akv;
+
+namespace {
+
+constexpr unsigned kPoison = 0x7fc00000u;
+
+// ---- norms of the two latents, rotation of the shared key part, cache write -------------------------------------------
+// One block per token.  down = [q latent | kv latent | key part]; the last two only where the layer keeps a cache.
+template <typename T>
+__global__ __launch_bounds__(256) void latent_encode_kernel(
+    const T* __restrict__ down, int q_rank, int kv_rank, int rot, int rot_dims, const float* __restrict__ q_weight,
+    const float* __restrict__ kv_weight, float eps, const float* __restrict__ table, int table_positions,
+    const int* __restrict__ positions, const int* __restrict__ slot_map, T* __restrict__ cq, T* __restrict__ records,
+    long record_slots) {
+  __shared__ float scratch[16];
+  const int n = blockIdx.x;
+  const bool writes = records != nullptr;
+  const int width = q_rank + (writes ? kv_rank + rot : 0);
+  const T* src = down + static_cast<size_t>(n) * width;
+  float acc = 0.f;
+  for (int i = threadIdx.x; i < q_rank; i += blockDim.x) {
+    const float v = to_float(src[i]);
+    acc += v * v;
+  }
+  const float q_scale = rsqrtf(block_sum(acc, scratch) / static_cast<float>(q_rank) + eps);
+  for (int i = threadIdx.x; i < q_rank; i += blockDim.x)
+    cq[static_cast<size_t>(n) * q_rank + i] = from_float<T>(to_float(src[i]) * q_scale * q_weight[i]);
+  if (!writes) return;
+  const long slot = slot_map[n];
+  if (slot < 0 || slot >= record_slots) return;     // (never write outside the pages)
+  T* record = records + slot * (kv_rank + rot);
+  const T* latent = src + q_rank;
+  acc = 0.f;
+  for (int i = threadIdx.x; i < kv_rank; i += blockDim.x) {
+    const float v = to_float(latent[i]);
+    acc += v * v;
+  }
+  const float kv_scale = rsqrtf(block_sum(acc, scratch) / static_cast<float>(kv_rank) + eps);
+  for (int i = threadIdx.x; i < kv_rank; i += blockDim.x)
+    record[i] = from_float<T>(to_float(latent[i]) * kv_scale * kv_weight[i]);
+  const T* key = latent + kv_rank;
+  const int half = rot_dims / 2;
+  const int pos = positions[n];
+  const bool known = pos >= 0 && pos < table_positions;
+  for (int i = threadIdx.x; i < rot; i += blockDim.x) {
+    float value;
+    if (i >= rot_dims) {
+      value = to_float(key[i]);
+    } else if (!known) {
+      value = __uint_as_float(kPoison);
+    } else {
+      const int j = i < half ? i : i - half;
+      const float c = table[(static_cast<size_t>(pos) * half + j) * 2], s = table[(static_cast<size_t>(pos) * half + j) * 2 + 1];
+      const float u = to_float(key[j]), v = to_float(key[j + half]);
+      value = i < half ? u * c - v * s : v * c + u * s;
+    }
+    record[kv_rank + i] = from_float<T>(value);
+  }
+}
+
+// ---- the rotated part of every query head, into its place behind the absorbed part --------------------------------------
+template <typename T>
+__global__ void rotate_queries_kernel(const T* __restrict__ q, long tokens, int heads, int dim, int rot, int rot_dims,
+                                      const float* __restrict__ table, int table_positions,
+                                      const int* __restrict__ positions, float* __restrict__ q_abs, int width, int at) {
+  const long index = static_cast<long>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (index >= tokens * heads * rot) return;
+  const int i = static_cast<int>(index % rot);
+  const long row = index / rot;                     // token * heads + head
+  const long n = row / heads;
+  const T* src = q + row * (dim + rot) + dim;
+  const int half = rot_dims / 2;
+  float value;
+  if (i >= rot_dims) {
+    value = to_float(src[i]);
+  } else {
+    const int pos = positions[n];
+    if (pos < 0 || pos >= table_positions) {
+      value = __uint_as_float(kPoison);
+    } else {
+      const int j = i < half ? i : i - half;
+      const float c = table[(static_cast<size_t>(pos) * half + j) * 2], s = table[(static_cast<size_t>(pos) * half + j) * 2 + 1];
+      const float u = to_float(src[j]), v = to_float(src[j + half]);
+      value = i < half ? u * c - v * s : v * c + u * s;
+    }
+  }
+  q_abs[row * width + at + i] = value;
+}
+
+// ---- y[t, h, j] = sum_i x[t, h, i] w[h, i, j] ------------------------------------------------------------------------------
+// A block takes kTokens tokens of one head and up to 256 outputs: thread j streams column j of the head's matrix
+// (neighbouring threads read neighbouring addresses) against the tokens' inputs, which lie in LDS as [i][token] so
+// that a thread reads the eight of an i as two 16-byte broadcasts.  Sums are float32 in the order of i whatever the
+// batch.
+constexpr int kHeadTokens = 8;
+
+template <typename TX, typename TW, typename TY>
+__global__ __launch_bounds__(256) void heads_linear_kernel(const TX* __restrict__ x, long x_token_stride,
+                                                           long x_head_stride, const TW* __restrict__ w,
+                                                           TY* __restrict__ y, long y_token_stride, long y_head_stride,
+                                                           int tokens, int ins, int outs) {
+  extern __shared__ float xs[];      // [ins][kHeadTokens]
+  const int h = blockIdx.y;
+  const int first = blockIdx.x * kHeadTokens;
+  const int j = blockIdx.z * blockDim.x + threadIdx.x;
+  for (int e = threadIdx.x; e < ins * kHeadTokens; e += blockDim.x) {
+    const int t = e / ins, i = e % ins;             // (consecutive threads read consecutive inputs of one token)
+    const int n = first + t;
+    xs[i * kHeadTokens + t] = n < tokens ? to_float(x[n * x_token_stride + h * x_head_stride + i]) : 0.f;
+  }
+  __syncthreads();
+  if (j >= outs) return;
+  const TW* column = w + static_cast<size_t>(h) * ins * outs + j;
+  float acc[kHeadTokens];
+#pragma unroll
+  for (int t = 0; t < kHeadTokens; ++t) acc[t] = 0.f;
+  for (int i = 0; i < ins; ++i) {
+    const float weight = to_float(column[static_cast<size_t>(i) * outs]);
+    const float4 a = *reinterpret_cast<const float4*>(xs + i * kHeadTokens);
+    const float4 b = *reinterpret_cast<const float4*>(xs + i * kHeadTokens + 4);
+    acc[0] = fmaf(a.x, weight, acc[0]);
+    acc[1] = fmaf(a.y, weight, acc[1]);
+    acc[2] = fmaf(a.z, weight, acc[2]);
+    acc[3] = fmaf(a.w, weight, acc[3]);
+    acc[4] = fmaf(b.x, weight, acc[4]);
+    acc[5] = fmaf(b.y, weight, acc[5]);
+    acc[6] = fmaf(b.z, weight, acc[6]);
+    acc[7] = fmaf(b.w, weight, acc[7]);
+  }
+#pragma unroll
+  for (int t = 0; t < kHeadTokens; ++t) {
+    const int n = first + t;
+    if (n < tokens) y[n * y_token_stride + h * y_head_stride + j] = from_float<TY>(acc[t]);
+  }
+}
+
+// ---- the attention itself ----------------------------------------------------------------------------------------------
+// A block is one token and up to eight heads, a wave each.  The records of KT keys at a time are fetched once for all
+// of the block's heads into LDS, as float32 rows an odd number of words apart.  Scores: a lane takes one key and one of
+// 64 / KT interleaved shares of the dimensions; the shares are added across lanes.  Weighted sum: a lane owns the
+// latent's dimensions lane, lane + 64, ...  Tiles are aligned to absolute key positions, so the order of every sum
+// depends on the token's position alone - not on the portion it arrived in, nor on what else is in the batch.
+constexpr int kMaxLatentRegs = 16;     // latents up to 1,024 wide
+
+template <typename T, int KT>
+__global__ __launch_bounds__(512) void latent_attend_kernel(
+    const float* __restrict__ q_abs, const T* __restrict__ records, const int* __restrict__ seq_of_token,
+    const int* __restrict__ positions, const int* __restrict__ block_table, const int* __restrict__ table_rows,
+    int table_width, float* __restrict__ out, int heads, int kv_rank, int width, int page_size, long num_pages,
+    float scale, int window) {
+  extern __shared__ float lds[];
+  constexpr int kShares = kWave / KT;
+  const int waves = blockDim.x / kWave, wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
+  const int padded = width | 1;
+  float* tile = lds;                                      // [KT][padded]
+  long* slot_of = reinterpret_cast<long*>(tile + KT * padded + (KT * padded & 1));   // [KT], -1: no such key
+  float* qs = reinterpret_cast<float*>(slot_of + KT) + wave * (width + KT);           // [width] and the weights [KT]
+  float* ps = qs + width;
+
+  const int n = blockIdx.x;
+  const int h = blockIdx.y * waves + wave;
+  const bool works = h < heads;
+  const int r = table_rows != nullptr ? table_rows[seq_of_token[n]] : seq_of_token[n];
+  const int pos = positions[n];
+  const int lowest = window > 0 ? max(0, pos - window + 1) : 0;
+  if (works)
+    for (int i = lane; i < width; i += kWave) qs[i] = q_abs[(static_cast<size_t>(n) * heads + h) * width + i];
+
+  const int key = lane % KT, share = lane / KT;
+  float m = -INFINITY, l = 0.f;
+  float acc[kMaxLatentRegs];
+#pragma unroll
+  for (int c = 0; c < kMaxLatentRegs; ++c) acc[c] = 0.f;
+  bool poisoned = false;
+
+  for (int t0 = lowest / KT * KT; t0 <= pos; t0 += KT) {
+    __syncthreads();                    // the tile of the turn before has been read by everybody
+    if (threadIdx.x < KT) {
+      const int j = t0 + threadIdx.x;
+      long slot = -1;
+      if (j >= lowest && j <= pos) {
+        const long page = block_table[static_cast<long>(r) * table_width + j / page_size];
+        slot = (page < 0 || page >= num_pages) ? -2 : page * page_size + j % page_size;   // -2: a page that is not the request's
+      }
+      slot_of[threadIdx.x] = slot;
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < KT * width; e += blockDim.x) {
+      const int k = e / width, i = e % width;
+      const long slot = slot_of[k];
+      tile[k * padded + i] = slot >= 0 ? to_float(records[slot * width + i]) : 0.f;
+    }
+    __syncthreads();
+    if (!works) continue;
+    const long slot = slot_of[key];
+    poisoned = poisoned || slot == -2;
+    float dot = 0.f;
+    const float* row = tile + key * padded;
+    for (int i = share; i < width; i += kShares) dot = fmaf(qs[i], row[i], dot);
+#pragma unroll
+    for (int offset = KT; offset < kWave; offset <<= 1) dot += __shfl_xor(dot, offset, kWave);
+    const float s = slot >= 0 ? dot * scale : -INFINITY;
+    const float m_new = fmaxf(m, wave_max(s));
+    const float p = slot >= 0 ? expf(s - m_new) : 0.f;
+    const float correction = expf(m - m_new);
+    l = l * correction + wave_sum(p) * (1.f / kShares);
+    m = m_new;
+    if (share == 0) ps[key] = p;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+    for (int c = 0; c < kMaxLatentRegs; ++c) acc[c] *= correction;
+    for (int k = 0; k < KT; ++k) {
+      const float pk = ps[k];
+      const float* value = tile + k * padded;
+#pragma unroll
+      for (int c = 0; c < kMaxLatentRegs; ++c) {
+        const int i = lane + c * kWave;
+        if (i < kv_rank) acc[c] = fmaf(pk, value[i], acc[c]);
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  }
+  if (!works) return;
+  // (any lane that met a foreign page poisons the head's output)
+  const bool any_poison = __any(poisoned);
+  float* dst = out + (static_cast<size_t>(n) * heads + h) * kv_rank;
+#pragma unroll
+  for (int c = 0; c < kMaxLatentRegs; ++c) {
+    const int i = lane + c * kWave;
+    if (i < kv_rank) dst[i] = any_poison ? __uint_as_float(kPoison) : acc[c] / l;
+  }
+}
+
+template <typename T, int KT>
+int launch_attend(const float* q_abs, const void* records, const int* seq_of_token, const int* positions,
+                  const int* block_table, const int* table_rows, int table_width, float* out, int tokens, int heads,
+                  int kv_rank, int width, int page_size, long num_pages, float scale, int window, int waves,
+                  size_t lds_bytes, hipStream_t stream) {
+  auto kernel = latent_attend_kernel<T, KT>;
+  if (lds_bytes > 64 * 1024 &&
+      hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                          static_cast<int>(lds_bytes)) != hipSuccess)
+    return -2;
+  kernel<<<dim3(tokens, (heads + waves - 1) / waves), waves * kWave, lds_bytes, stream>>>(
+      q_abs, static_cast<const T*>(records), seq_of_token, positions, block_table, table_rows, table_width, out, heads,
+      kv_rank, width, page_size, num_pages, scale, window);
+  return AKV_LAUNCH_STATUS();
+}
+
+size_t attend_lds(int kt, int width, int waves) {
+  const size_t padded = width | 1;
+  size_t floats = kt * padded;
+  floats += floats & 1;
+  return floats * 4 + static_cast<size_t>(kt) * 8 + static_cast<size_t>(waves) * (width + kt) * 4;
+}
+
+}  // namespace
+
+extern "C" {
+
+int akv_latent_encode(const void* down, int dtype, int tokens, int q_rank, int kv_rank, int rot, int rot_dims,
+                      const float* q_weight, const float* kv_weight, float eps, const float* table, int table_positions,
+                      const int* positions, const int* slot_map, void* cq, void* records, long record_slots,
+                      hipStream_t stream) {
+  if (tokens <= 0) return 0;
+  if (rot_dims % 2 || rot_dims > rot || q_rank <= 0) return -2;
+  AKV_DISPATCH(dtype, T, latent_encode_kernel<T><<<tokens, 256, 0, stream>>>(
+                             static_cast<const T*>(down), q_rank, kv_rank, rot, rot_dims, q_weight, kv_weight, eps, table,
+                             table_positions, positions, slot_map, static_cast<T*>(cq), static_cast<T*>(records),
+                             record_slots));
+  return AKV_LAUNCH_STATUS();
+}
+
+int akv_rotate_queries(const void* q, int dtype, long tokens, int heads, int dim, int rot, int rot_dims,
+                       const float* table, int table_positions, const int* positions, float* q_abs, int width, int at,
+                       hipStream_t stream) {
+  const long count = tokens * heads * rot;
+  if (count <= 0) return 0;
+  if (rot_dims % 2 || rot_dims > rot || at + rot > width) return -2;
+  AKV_DISPATCH(dtype, T, rotate_queries_kernel<T><<<static_cast<unsigned>((count + 255) / 256), 256, 0, stream>>>(
+                             static_cast<const T*>(q), tokens, heads, dim, rot, rot_dims, table, table_positions, positions,
+                             q_abs, width, at));
+  return AKV_LAUNCH_STATUS();
+}
+
+int akv_heads_linear(const void* x, int x_dtype, long x_token_stride, long x_head_stride, const void* w, int w_dtype,
+                     void* y, int y_dtype, long y_token_stride, long y_head_stride, int tokens, int heads, int ins,
+                     int outs, hipStream_t stream) {
+  if (tokens <= 0 || heads <= 0) return 0;
+  if (ins <= 0 || outs <= 0) return -2;
+  const size_t lds_bytes = static_cast<size_t>(ins) * kHeadTokens * 4;
+  if (lds_bytes > 64 * 1024) return -2;
+  const int threads = outs >= 256 ? 256 : (outs + kWave - 1) / kWave * kWave;
+  const dim3 grid((tokens + kHeadTokens - 1) / kHeadTokens, heads, (outs + threads - 1) / threads);
+#define AKV_HEADS(TX, TW, TY)                                                                                       \
+  heads_linear_kernel<TX, TW, TY><<<grid, threads, lds_bytes, stream>>>(                                            \
+      static_cast<const TX*>(x), x_token_stride, x_head_stride, static_cast<const TW*>(w), static_cast<TY*>(y),    \
+      y_token_stride, y_head_stride, tokens, ins, outs)
+  if (x_dtype == kF32 && w_dtype == kF32 && y_dtype == kF32) AKV_HEADS(float, float, float);
+  else if (x_dtype == kBF16 && w_dtype == kBF16 && y_dtype == kF32) AKV_HEADS(bf16_t, bf16_t, float);
+  else if (x_dtype == kF32 && w_dtype == kBF16 && y_dtype == kBF16) AKV_HEADS(float, bf16_t, bf16_t);
+  else if (x_dtype == kF32 && w_dtype == kBF16 && y_dtype == kF32) AKV_HEADS(float, bf16_t, float);
+  else return -1;
+#undef AKV_HEADS
+  return AKV_LAUNCH_STATUS();
+}
+
+int akv_latent_attend(const float* q_abs, const void* records, int dtype, const int* seq_of_token, const int* positions,
+                      const int* block_table, const int* table_rows, int table_width, float* out, int tokens, int heads,
+                      int kv_rank, int width, int page_size, long num_pages, float scale, int window,
+                      hipStream_t stream) {
+  if (tokens <= 0) return 0;
+  if (kv_rank <= 0 || kv_rank > width || kv_rank > kMaxLatentRegs * kWave || page_size <= 0) return -2;
+  const int waves = heads < 8 ? heads : 8;
+  // the most keys a turn whose records, beside the heads' queries, fit the 64 KB every block may ask for
+  int kt = 64;
+  while (kt > 8 && attend_lds(kt, width, waves) > 64 * 1024) kt >>= 1;
+  const size_t lds_bytes = attend_lds(kt, width, waves);
+  if (lds_bytes > device_facts().lds_bytes) return -2;
+#define AKV_ATTEND(T, KT)                                                                                               \
+  return launch_attend<T, KT>(q_abs, records, seq_of_token, positions, block_table, table_rows, table_width, out, tokens, \
+                              heads, kv_rank, width, page_size, num_pages, scale, window, waves, lds_bytes, stream)
+  AKV_DISPATCH(dtype, T, {
+    if (kt == 64) AKV_ATTEND(T, 64);
+    if (kt == 32) AKV_ATTEND(T, 32);
+    if (kt == 16) AKV_ATTEND(T, 16);
+    AKV_ATTEND(T, 8);
+  });
+#undef AKV_ATTEND
+  return -2;
+}
+}

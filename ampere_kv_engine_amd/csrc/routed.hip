@@ -1,0 +1,118 @@
+// A routed feed-forward's token-wise kernels: the router (float32 logits, softmax over all experts, the choice
+// restricted to the best groups of neighbouring experts) and the experts' activation times the router's weight.
+
+#include "common.h"
+#include "api_parts.h"
+
+using namespace akv;
+
+namespace {
+
+// One wave per token.  scores = softmax(router x); a group's score is its best expert's; only experts of the `keep`
+// best groups can be chosen; the `top` best of those are, each weighted by its own score (the weights are not
+// renormalised).  Equal scores go to the lower index.  gates[t, e] = score of a chosen expert, 0 of any other.
+template <typename T>
+__global__ __launch_bounds__(256) void route_kernel(const T* __restrict__ x, const float* __restrict__ router,
+                                                    float* __restrict__ gates, int tokens, int hidden, int experts,
+                                                    int top, int groups, int keep) {
+  extern __shared__ float lds[];
+  const int waves = blockDim.x / kWave, wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
+  const int n = blockIdx.x * waves + wave;
+  if (n >= tokens) return;
+  float* score = lds + static_cast<size_t>(wave) * (2 * experts + groups);   // [experts]
+  float* open = score + experts;        // [experts]: 1 while the expert may still be chosen, 2 once it is chosen, 0 shut
+  float* best = open + experts;         // [groups]
+  const T* row = x + static_cast<size_t>(n) * hidden;
+  for (int e = 0; e < experts; ++e) {
+    const float* w = router + static_cast<size_t>(e) * hidden;
+    float acc = 0.f;
+    for (int i = lane; i < hidden; i += kWave) acc = fmaf(to_float(row[i]), w[i], acc);
+    acc = wave_sum(acc);
+    if (lane == 0) score[e] = acc;
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  if (lane == 0) {       // a few dozen numbers: one lane does the choosing
+    float highest = -INFINITY, total = 0.f;
+    for (int e = 0; e < experts; ++e) highest = fmaxf(highest, score[e]);
+    for (int e = 0; e < experts; ++e) {
+      score[e] = expf(score[e] - highest);
+      total += score[e];
+    }
+    const int size = experts / groups;
+    for (int e = 0; e < experts; ++e) {
+      score[e] = score[e] / total;
+      open[e] = 0.f;
+    }
+    for (int g = 0; g < groups; ++g) {
+      float top_of = -INFINITY;
+      for (int e = g * size; e < (g + 1) * size; ++e) top_of = fmaxf(top_of, score[e]);
+      best[g] = top_of;
+    }
+    for (int k = 0; k < keep; ++k) {
+      int at = -1;
+      for (int g = 0; g < groups; ++g)
+        if (best[g] >= 0.f && (at < 0 || best[g] > best[at])) at = g;
+      if (at < 0) break;
+      best[at] = -1.f;              // (scores are never negative)
+      for (int e = at * size; e < (at + 1) * size; ++e) open[e] = 1.f;
+    }
+    for (int k = 0; k < top; ++k) {
+      int at = -1;
+      for (int e = 0; e < experts; ++e)
+        if (open[e] == 1.f && (at < 0 || score[e] > score[at])) at = e;
+      if (at < 0) break;
+      open[at] = 2.f;
+    }
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  for (int e = lane; e < experts; e += kWave) gates[static_cast<size_t>(n) * experts + e] = open[e] == 2.f ? score[e] : 0.f;
+}
+
+// act[t, e * ff + j] = gates[t, e] * relu(up[t, e * ff + j])^2, formed in float32 and rounded once; an expert that was
+// not chosen gives exact zeros whatever its product holds.
+template <typename T>
+__global__ void gate_relu_squared_kernel(const T* __restrict__ up, const float* __restrict__ gates, T* __restrict__ act,
+                                         long tokens, int experts, int ff) {
+  const long index = static_cast<long>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const long width = static_cast<long>(experts) * ff;
+  if (index >= tokens * width) return;
+  const long n = index / width;
+  const int e = static_cast<int>((index % width) / ff);
+  const float g = gates[n * experts + e];
+  float value = 0.f;
+  if (g != 0.f) {
+    const float u = fmaxf(to_float(up[index]), 0.f);
+    value = g * (u * u);
+  }
+  act[index] = from_float<T>(value);
+}
+
+}  // namespace
+
+extern "C" {
+
+int akv_route(const void* x, int dtype, const float* router, float* gates, int tokens, int hidden, int experts,
+              int top, int groups, int keep, hipStream_t stream) {
+  if (tokens <= 0) return 0;
+  if (experts <= 0 || groups <= 0 || experts % groups || keep <= 0 || keep > groups || top <= 0 || top > experts) return -2;
+  const int waves = 4;
+  const size_t lds_bytes = static_cast<size_t>(waves) * (2 * experts + groups) * 4;
+  if (lds_bytes > 64 * 1024) return -2;
+  AKV_DISPATCH(dtype, T, route_kernel<T><<<(tokens + waves - 1) / waves, waves * kWave, lds_bytes, stream>>>(
+                             static_cast<const T*>(x), router, gates, tokens, hidden, experts, top, groups, keep));
+  return AKV_LAUNCH_STATUS();
+}
+
+int akv_gate_relu_squared(const void* up, const float* gates, void* act, int dtype, long tokens, int experts, int ff,
+                          hipStream_t stream) {
+  const long count = tokens * experts * ff;
+  if (count <= 0) return 0;
+  AKV_DISPATCH(dtype, T, gate_relu_squared_kernel<T><<<static_cast<unsigned>((count + 255) / 256), 256, 0, stream>>>(
+                             static_cast<const T*>(up), gates, static_cast<T*>(act), tokens, experts, ff));
+  return AKV_LAUNCH_STATUS();
+}
+}

@@ -1,0 +1,137 @@
+// Token-wise kernels of designs whose norms and residual sum are float32 from end to end: an embedding that adds a row
+// of a hashed table of token pairs, and the norm kernel of blocks that norm every branch before AND after.  Nothing
+// is rounded between a sum of squares and the one store of a result.
+
+#include "common.h"
+#include "api_parts.h"
+
+using namespace akv;
+
+namespace {
+
+constexpr unsigned kPoison = 0x7fc00000u;
+
+// ---- embedding plus a row of the pair table ---------------------------------------------------------------------------
+// The pair of a portion's first token reaches back into the previous step: the request's slot keeps the id it was
+// fed last (kSlotFedToken), written by note_fed_tokens_kernel after this kernel has read it.
+template <typename T>
+__global__ __launch_bounds__(256) void embed_pairs_kernel(
+    const int* __restrict__ ids, const T* __restrict__ table, const T* __restrict__ pairs, float* __restrict__ out,
+    int hidden, int vocab, long buckets, long mul_prev, long mul_cur, const int* __restrict__ seq_of_token,
+    const int* __restrict__ q_start, const int* __restrict__ positions, const int* __restrict__ seq_slots,
+    const int* __restrict__ slot_words) {
+  const int n = blockIdx.x;
+  const int r = seq_of_token[n];
+  const long slot = seq_slots[r];
+  int id = ids[n];
+  if (id == -1) id = slot_words[slot * kSlotWords + kSlotLastToken];
+  long pair_row = buckets;                   // a request's first token: the table's last row
+  bool bad = id < 0 || id >= vocab;
+  if (positions[n] > 0) {
+    const int prev = n > q_start[r] ? ids[n - 1] : slot_words[slot * kSlotWords + kSlotFedToken];
+    bad = bad || prev < 0 || prev >= vocab;
+    const long mixed = (static_cast<long>(prev) * mul_prev + static_cast<long>(id) * mul_cur) % buckets;
+    pair_row = mixed < 0 ? mixed + buckets : mixed;
+  }
+  float* dst = out + static_cast<size_t>(n) * hidden;
+  if (bad) {     // never read outside a table; a poisoned row shows the fault downstream
+    for (int d = threadIdx.x; d < hidden; d += blockDim.x) dst[d] = __uint_as_float(kPoison);
+    return;
+  }
+  const T* token_row = table + static_cast<size_t>(id) * hidden;
+  const T* pair = pairs + static_cast<size_t>(pair_row) * hidden;
+  for (int d = threadIdx.x; d < hidden; d += blockDim.x) dst[d] = to_float(token_row[d]) + to_float(pair[d]);
+}
+
+__global__ void note_fed_tokens_kernel(const int* __restrict__ ids, const int* __restrict__ q_start,
+                                       const int* __restrict__ seq_slots, int* __restrict__ slot_words, int seqs) {
+  const int r = blockIdx.x * blockDim.x + threadIdx.x;
+  if (r >= seqs) return;
+  const long slot = seq_slots[r];
+  int id = ids[q_start[r + 1] - 1];
+  if (id == -1) id = slot_words[slot * kSlotWords + kSlotLastToken];
+  slot_words[slot * kSlotWords + kSlotFedToken] = id;
+}
+
+// ---- stream += norm_post(delta); out = norm_pre(stream) -----------------------------------------------------------------
+// One block per row, three passes over a row that the caches hold: the branch's sum of squares; the update of the
+// residual sum, which gathers the new sum of squares as it goes; the normed row.
+template <typename T>
+__global__ __launch_bounds__(256) void norm_add_norm_kernel(float* __restrict__ stream, const T* __restrict__ delta,
+                                                            const float* __restrict__ post_weight, float post_eps,
+                                                            const float* __restrict__ pre_weight, float pre_eps,
+                                                            T* __restrict__ out, int hidden) {
+  __shared__ float scratch[16];
+  const size_t base = static_cast<size_t>(blockIdx.x) * hidden;
+  float* s = stream + base;
+  float squares = 0.f;
+  if (delta != nullptr) {
+    const T* d = delta + base;
+    float post_scale = 1.f;
+    if (post_weight != nullptr) {
+      float acc = 0.f;
+      for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+        const float v = to_float(d[i]);
+        acc += v * v;
+      }
+      post_scale = rsqrtf(block_sum(acc, scratch) / static_cast<float>(hidden) + post_eps);
+    }
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+      const float add = post_weight != nullptr ? to_float(d[i]) * post_scale * post_weight[i] : to_float(d[i]);
+      const float v = s[i] + add;
+      s[i] = v;
+      squares += v * v;
+    }
+  } else if (out != nullptr) {
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+      const float v = s[i];
+      squares += v * v;
+    }
+  }
+  if (out == nullptr) return;
+  const float scale = rsqrtf(block_sum(squares, scratch) / static_cast<float>(hidden) + pre_eps);
+  T* o = out + base;
+  // (a thread reads back what it wrote itself: the same elements in every pass)
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) o[i] = from_float<T>(s[i] * scale * pre_weight[i]);
+}
+
+}  // namespace
+
+extern "C" {
+
+int akv_parts_slot_layout(int* out) {
+  out[0] = kSlotWords;
+  out[1] = kSlotLastToken;
+  out[2] = kSlotFedToken;
+  return 0;
+}
+
+int akv_embed_pairs(const int* ids, const void* table, const void* pairs, int dtype, float* out, int tokens, int hidden,
+                    int vocab, long buckets, long mul_prev, long mul_cur, const int* seq_of_token, const int* q_start,
+                    const int* positions, const int* seq_slots, int* slot_words, hipStream_t stream) {
+  if (tokens <= 0) return 0;
+  if (buckets <= 0) return -2;
+  AKV_DISPATCH(dtype, T, embed_pairs_kernel<T><<<tokens, 256, 0, stream>>>(
+                             ids, static_cast<const T*>(table), static_cast<const T*>(pairs), out, hidden, vocab, buckets,
+                             mul_prev, mul_cur, seq_of_token, q_start, positions, seq_slots, slot_words));
+  return AKV_LAUNCH_STATUS();
+}
+
+int akv_note_fed_tokens(const int* ids, const int* q_start, const int* seq_slots, int* slot_words, int seqs,
+                        hipStream_t stream) {
+  if (seqs <= 0) return 0;
+  note_fed_tokens_kernel<<<(seqs + 63) / 64, 64, 0, stream>>>(ids, q_start, seq_slots, slot_words, seqs);
+  return AKV_LAUNCH_STATUS();
+}
+
+int akv_norm_add_norm(float* stream_buf, const void* delta, const float* post_weight, float post_eps,
+                      const float* pre_weight, float pre_eps, void* out, int dtype, int tokens, int hidden,
+                      hipStream_t stream) {
+  if (tokens <= 0) return 0;
+  if (out != nullptr && pre_weight == nullptr) return -2;
+  AKV_DISPATCH(dtype, T, norm_add_norm_kernel<T><<<tokens, 256, 0, stream>>>(
+                             stream_buf, static_cast<const T*>(delta), post_weight, post_eps, pre_weight, pre_eps,
+                             static_cast<T*>(out), hidden));
+  return AKV_LAUNCH_STATUS();
+}
+}

@@ -20,7 +20,7 @@ import sys
 
 import numpy as np
 
-MAX_LIVE_REQUESTS = 8
+MAX_LIVE_REQUESTS = 4   # request slots of a replay's engine: freed slots and pages come round again within a trace
 PAGE_SIZE = 16
 ROUND_TOKENS = 64       # `--max-tokens` counts every live request rounded up to a multiple of this many tokens
 

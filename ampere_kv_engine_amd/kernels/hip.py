@@ -13,6 +13,7 @@ import torch
 
 from ..csrc.build import ensure_attention, ensure_built
 from ..parts.base import KernelSet
+from .hip_parts import PartsKernels
 
 _DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
 MAX_HEAD_DIM = 256
@@ -87,7 +88,7 @@ def _ptr(t: torch.Tensor | None):
     return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
 
 
-class HipKernels(KernelSet):
+class HipKernels(PartsKernels, KernelSet):
     name = "hip-gfx950"
     OWN_SKINNY_ROWS = 64            # the most rows the engine's own decode product takes
 

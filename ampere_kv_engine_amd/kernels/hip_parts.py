@@ -1,0 +1,280 @@
+"""Wrappers over the second kernel library (`csrc/api_parts.h`): the token-wise kernels, mixers and routed feed-forward
+of designs whose norms and residual sum are float32 throughout.  `HipKernels` inherits them; the library is compiled
+and loaded when a model first asks for one of them.  As everywhere in the kernel set, shapes, dtypes, contiguity and
+devices are checked on the host before a launch."""
+
+from __future__ import annotations
+
+import ctypes
+
+import torch
+
+from ..csrc.build import ensure_parts
+
+_DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
+
+
+def _long(value: int):
+    return ctypes.c_long(int(value))
+
+
+class PartsKernels:
+    """Mixed into `HipKernels` (which provides `_dense`, `_check`, `_stream`, `device`)."""
+
+    _parts_lib = None
+
+    def _parts(self):
+        if self._parts_lib is None:
+            from ..cache import slots
+            from .hip import KernelError
+            path = ensure_parts()
+            try:
+                lib = ctypes.CDLL(path)
+            except OSError as error:
+                raise KernelError(f"the kernel library {path} could not be loaded: {error}") from error
+            for name in ("akv_embed_pairs", "akv_note_fed_tokens", "akv_norm_add_norm", "akv_latent_encode",
+                         "akv_rotate_queries", "akv_heads_linear", "akv_latent_attend", "akv_conv_silu",
+                         "akv_conv_state_update", "akv_selective_scan", "akv_route", "akv_gate_relu_squared",
+                         "akv_parts_slot_layout"):
+                getattr(lib, name).restype = ctypes.c_int
+            layout = (ctypes.c_int * 3)()
+            lib.akv_parts_slot_layout(layout)
+            if tuple(layout) != (slots.SLOT_WORDS, slots.WORD_LAST_TOKEN, slots.WORD_FED_TOKEN):
+                raise KernelError(f"the kernel library lays a request's slot out as {tuple(layout)} (words, last token, "
+                                  "fed token); the host otherwise")
+            self._parts_lib = lib
+            self.parts_library_path = path
+        return self._parts_lib
+
+    def _code_of(self, t: torch.Tensor) -> int:
+        from .hip import KernelError
+        try:
+            return _DTYPE_CODE[t.dtype]
+        except KeyError:
+            raise KernelError(f"kernels take float32 or bfloat16 tensors, got {t.dtype}") from None
+
+    def _refuse(self, message: str):
+        from .hip import KernelError
+        raise KernelError(message)
+
+    def _step_arrays(self, ctx, tokens: int):
+        self._dense(ctx.seq_of_token, "seq_of_token", torch.int32, (tokens,))
+        self._dense(ctx.q_start, "q_start", torch.int32, (ctx.num_seqs + 1,))
+        self._dense(ctx.seq_slots, "seq_slots", torch.int32, (ctx.num_seqs,))
+        self._dense(ctx.positions, "positions", torch.int32, (tokens,))
+        if ctx.host_q_start[-1] != tokens:
+            self._refuse("the step's request boundaries do not end at its last token")
+
+    # ---- token-wise ------------------------------------------------------------------------------------------------------
+    def embed_pairs(self, ids, table, pairs, buckets: int, mul_prev: int, mul_cur: int, out, ctx) -> None:
+        """out[n] = table[id] + pairs[(previous id * mul_prev + id * mul_cur) mod buckets] (row `buckets` for a request's
+        first token); the id a request was fed last is kept in its slot for the next step's first pair."""
+        lib = self._parts()
+        tokens = ids.shape[0]
+        vocab, hidden = table.shape
+        self._dense(ids, "ids", torch.int32, (tokens,))
+        self._dense(table, "table")
+        self._dense(pairs, "pairs", table.dtype, (buckets + 1, hidden))
+        self._dense(out, "out", torch.float32, (tokens, hidden))
+        words = getattr(ctx, "slot_words", None)
+        if words is None:
+            self._refuse("an embedding of token pairs needs the requests' slots (the token each was fed last)")
+        self._dense(words, "slot_words", torch.int32)
+        self._step_arrays(ctx, tokens)
+        if max(ctx.host_seq_slots) >= words.shape[0]:
+            self._refuse("a request's slot lies outside the slot words")
+        self._check(lib.akv_embed_pairs(_ptr(ids), _ptr(table), _ptr(pairs), self._code_of(table), _ptr(out), tokens, hidden,
+                                        vocab, _long(buckets), _long(mul_prev), _long(mul_cur), _ptr(ctx.seq_of_token),
+                                        _ptr(ctx.q_start), _ptr(ctx.positions), _ptr(ctx.seq_slots), _ptr(words),
+                                        self._stream()), "embed_pairs")
+        self._check(lib.akv_note_fed_tokens(_ptr(ids), _ptr(ctx.q_start), _ptr(ctx.seq_slots), _ptr(words), ctx.num_seqs,
+                                            self._stream()), "note_fed_tokens")
+
+    def norm_add_norm(self, stream, delta, post_weight, post_eps, pre_weight, pre_eps, out) -> None:
+        """stream (float32) += delta / rms(delta) * post_weight (+= delta where `post_weight` is None; nothing where
+        `delta` is None); then, where `out` is given, out = stream / rms(stream) * pre_weight.  Float32 up to the one
+        rounding of a stored result."""
+        tokens, hidden = stream.shape
+        self._dense(stream, "stream", torch.float32)
+        dtype = None
+        if delta is not None:
+            self._dense(delta, "delta", None, (tokens, hidden))
+            dtype = delta.dtype
+        if out is not None:
+            self._dense(out, "out", dtype, (tokens, hidden))
+            self._dense(pre_weight, "pre_weight", torch.float32, (hidden,))
+            dtype = out.dtype
+        if post_weight is not None:
+            self._dense(post_weight, "post_weight", torch.float32, (hidden,))
+        if dtype is None:
+            return
+        self._check(self._parts().akv_norm_add_norm(_ptr(stream), _ptr(delta), _ptr(post_weight), ctypes.c_float(post_eps),
+                                                    _ptr(pre_weight), ctypes.c_float(pre_eps), _ptr(out), _DTYPE_CODE[dtype],
+                                                    tokens, hidden, self._stream()), "norm_add_norm")
+
+    # ---- attention over a compressed latent --------------------------------------------------------------------------
+    def latent_encode(self, down, q_rank, kv_rank, rot, rot_dims, q_weight, kv_weight, eps, table, positions, slot_map,
+                      cq, records) -> None:
+        """down [tokens, q_rank (+ kv_rank + rot)] -> cq = norm(q latent); with `records` [pages, 1, page, kv_rank + rot]
+        also the token's record: norm(kv latent), then the key part with its first `rot_dims` dimensions rotated."""
+        tokens = down.shape[0]
+        writes = records is not None
+        self._dense(down, "down", None, (tokens, q_rank + (kv_rank + rot if writes else 0)))
+        self._dense(cq, "cq", down.dtype, (tokens, q_rank))
+        self._dense(q_weight, "q_weight", torch.float32, (q_rank,))
+        self._dense(positions, "positions", torch.int32, (tokens,))
+        slots = 0
+        if writes:
+            self._dense(records, "records", down.dtype)
+            if records.dim() != 4 or records.shape[1] != 1 or records.shape[3] != kv_rank + rot:
+                self._refuse(f"records must be [pages, 1, page, {kv_rank + rot}], got {tuple(records.shape)}")
+            slots = records.shape[0] * records.shape[2]
+            self._dense(kv_weight, "kv_weight", torch.float32, (kv_rank,))
+            self._dense(slot_map, "slot_map", torch.int32, (tokens,))
+            self._dense(table, "table", torch.float32)
+            if table.dim() != 3 or table.shape[1] != rot_dims // 2 or table.shape[2] != 2:
+                self._refuse(f"the rotation table must be [positions, {rot_dims // 2}, 2], got {tuple(table.shape)}")
+        self._check(self._parts().akv_latent_encode(
+            _ptr(down), self._code_of(down), tokens, q_rank, kv_rank, rot, rot_dims, _ptr(q_weight), _ptr(kv_weight),
+            ctypes.c_float(eps), _ptr(table) if writes else ctypes.c_void_p(0), table.shape[0] if writes else 0,
+            _ptr(positions), _ptr(slot_map) if writes else ctypes.c_void_p(0), _ptr(cq),
+            _ptr(records) if writes else ctypes.c_void_p(0), _long(slots), self._stream()), "latent_encode")
+
+    def rotate_queries(self, q, heads, dim, rot, rot_dims, table, positions, q_abs, at) -> None:
+        """q [tokens, heads * (dim + rot)] -> q_abs[:, :, at:at + rot] (float32): every head's last `rot` dimensions,
+        the first `rot_dims` of them rotated by the token's position."""
+        tokens = q.shape[0]
+        self._dense(q, "q", None, (tokens, heads * (dim + rot)))
+        self._dense(q_abs, "q_abs", torch.float32)
+        if q_abs.dim() != 3 or q_abs.shape[0] != tokens or q_abs.shape[1] != heads or at + rot > q_abs.shape[2]:
+            self._refuse(f"q_abs must be [tokens, heads, at least {at + rot}], got {tuple(q_abs.shape)}")
+        self._dense(table, "table", torch.float32)
+        if table.dim() != 3 or table.shape[1] != rot_dims // 2 or table.shape[2] != 2:
+            self._refuse(f"the rotation table must be [positions, {rot_dims // 2}, 2], got {tuple(table.shape)}")
+        self._dense(positions, "positions", torch.int32, (tokens,))
+        self._check(self._parts().akv_rotate_queries(_ptr(q), self._code_of(q), _long(tokens), heads, dim, rot, rot_dims,
+                                                     _ptr(table), table.shape[0], _ptr(positions), _ptr(q_abs),
+                                                     q_abs.shape[2], at, self._stream()), "rotate_queries")
+
+    def heads_linear(self, x, x_width: int, weight, y, y_width: int) -> None:
+        """y[t, h, :outs] = x[t, h, :ins] W[h] for W [heads, ins, outs]: `x` is [tokens, heads, x_width] and `y`
+        [tokens, heads, y_width], of which the product reads the first `ins` and writes the first `outs` of every head."""
+        heads, ins, outs = weight.shape
+        tokens = x.shape[0]
+        self._dense(weight, "weight")
+        self._dense(x, "x", None, (tokens, heads, x_width))
+        self._dense(y, "y", None, (tokens, heads, y_width))
+        if ins > x_width or outs > y_width:
+            self._refuse(f"a product of {ins} -> {outs} per head does not fit rows of {x_width} and {y_width}")
+        self._check(self._parts().akv_heads_linear(
+            _ptr(x), self._code_of(x), _long(heads * x_width), _long(x_width), _ptr(weight), self._code_of(weight), _ptr(y),
+            self._code_of(y), _long(heads * y_width), _long(y_width), tokens, heads, ins, outs, self._stream()),
+            "heads_linear")
+
+    def latent_attend(self, q_abs, records, ctx, meta, heads, kv_rank, scale, window, out) -> None:
+        """Every head of every token attends the records [kv_rank + rot] of its request's last `window` tokens (all,
+        if None): softmax((q_abs . record) * scale), then the weighted sum of the records' first kv_rank dimensions
+        -> out [tokens, heads, kv_rank] float32."""
+        tokens, width = q_abs.shape[0], q_abs.shape[2]
+        self._dense(q_abs, "q_abs", torch.float32, (tokens, heads, width))
+        self._dense(out, "out", torch.float32, (tokens, heads, kv_rank))
+        self._dense(records, "records")
+        if records.dim() != 4 or records.shape[1] != 1 or records.shape[3] != width:
+            self._refuse(f"records must be [pages, 1, page, {width}], got {tuple(records.shape)}")
+        self._dense(meta.block_table, "block_table", torch.int32)
+        if meta.block_table.dim() != 2 or meta.block_table.shape[1] != meta.width:
+            self._refuse("the block table does not have the width the step names")
+        self._step_arrays(ctx, tokens)
+        if meta.rows is not None:
+            self._dense(meta.rows, "table rows", torch.int32, (ctx.num_seqs,))
+            if max(ctx.host_seq_slots) >= meta.block_table.shape[0]:
+                self._refuse("a request's slot lies outside the block table")
+        elif ctx.num_seqs > meta.block_table.shape[0]:
+            self._refuse("the block table has fewer rows than the step has requests")
+        if ctx.max_seq_len > meta.width * records.shape[2]:
+            self._refuse("a request is longer than its row of the block table")
+        self._check(self._parts().akv_latent_attend(
+            _ptr(q_abs), _ptr(records), self._code_of(records), _ptr(ctx.seq_of_token), _ptr(ctx.positions),
+            _ptr(meta.block_table), _ptr(meta.rows), meta.width, _ptr(out), tokens, heads, kv_rank, width, records.shape[2],
+            _long(records.shape[0]), ctypes.c_float(scale), int(window) if window is not None else 0, self._stream()),
+            "latent_attend")
+
+    # ---- selective scan ------------------------------------------------------------------------------------------------
+    def _scan_state(self, state, ctx, channels, n_state, taps):
+        self._dense(state, "state", torch.float32)
+        need = channels * n_state + (taps - 1) * channels
+        if state.dim() != 2 or state.shape[1] != need:
+            self._refuse(f"the scan's state must be [slots, {need}], got {tuple(state.shape)}")
+        if max(ctx.host_seq_slots) >= state.shape[0]:
+            self._refuse("a request's slot lies outside the state")
+
+    def conv_silu(self, xz, channels, weight, bias, state, n_state, ctx, out) -> None:
+        """out[t, c] = silu(bias[c] + sum_k weight[c, k] * x[t - (taps - 1 - k), c]) over the first `channels` columns
+        of `xz`; inputs before a portion come from the request's state (zeros before its first token).  Afterwards the
+        state holds the last taps - 1 inputs of every request of the step."""
+        tokens, taps = xz.shape[0], weight.shape[1]
+        self._dense(xz, "xz")
+        if xz.dim() != 2 or xz.shape[1] < channels:
+            self._refuse(f"xz must be [tokens, at least {channels}], got {tuple(xz.shape)}")
+        self._dense(weight, "weight", None, (channels, taps))
+        self._dense(bias, "bias", weight.dtype, (channels,))
+        self._dense(out, "out", xz.dtype, (tokens, channels))
+        self._scan_state(state, ctx, channels, n_state, taps)
+        self._step_arrays(ctx, tokens)
+        lib, conv_at = self._parts(), channels * n_state
+        self._check(lib.akv_conv_silu(_ptr(xz), _long(xz.shape[1]), self._code_of(xz), _ptr(weight), _ptr(bias),
+                                      self._code_of(weight), _ptr(state), _long(state.shape[1]), _long(conv_at),
+                                      _ptr(ctx.seq_of_token), _ptr(ctx.q_start), _ptr(ctx.seq_slots), _ptr(out), tokens,
+                                      channels, taps, self._stream()), "conv_silu")
+        self._check(lib.akv_conv_state_update(_ptr(xz), _long(xz.shape[1]), self._code_of(xz), _ptr(state),
+                                              _long(state.shape[1]), _long(conv_at), _ptr(ctx.q_start), _ptr(ctx.seq_slots),
+                                              ctx.num_seqs, channels, taps, self._stream()), "conv_state_update")
+
+    def selective_scan(self, x, dt, bc, xz, a, d, state, taps, ctx, out) -> None:
+        """Per request and channel, token after token: S <- exp(softplus(dt) A) S + softplus(dt) x B, y = S C + D x,
+        out = y * silu(z), with z the second half of `xz`'s columns and S [channels, n_state] at the start of the
+        request's state (read at the portion's start, written back at its end)."""
+        tokens, channels = x.shape
+        n_state = a.shape[1]
+        self._dense(x, "x", None, (tokens, channels))
+        self._dense(dt, "dt", torch.float32, (tokens, channels))
+        self._dense(bc, "bc", torch.float32, (tokens, 2 * n_state))
+        self._dense(xz, "xz", x.dtype, (tokens, 2 * channels))
+        self._dense(a, "a", torch.float32, (channels, n_state))
+        self._dense(d, "d", torch.float32, (channels,))
+        self._dense(out, "out", x.dtype, (tokens, channels))
+        self._scan_state(state, ctx, channels, n_state, taps)
+        self._step_arrays(ctx, tokens)
+        z = xz[:, channels:]
+        self._check(self._parts().akv_selective_scan(
+            _ptr(x), self._code_of(x), _ptr(dt), _ptr(bc), ctypes.c_void_p(z.data_ptr()), _long(2 * channels), _ptr(a),
+            _ptr(d), _ptr(state), _long(state.shape[1]), _ptr(ctx.q_start), _ptr(ctx.seq_slots), _ptr(out), ctx.num_seqs,
+            channels, n_state, self._stream()), "selective_scan")
+
+    # ---- routed feed-forward -------------------------------------------------------------------------------------------
+    def route(self, x, router, gates, top: int, groups: int, keep: int) -> None:
+        """gates[t, e] = softmax(router x_t)[e] for the `top` best experts among those of the `keep` best of `groups`
+        groups of neighbouring experts (a group's score is its best expert's), 0 for every other expert."""
+        tokens, hidden = x.shape
+        experts = router.shape[0]
+        self._dense(x, "x")
+        self._dense(router, "router", torch.float32, (experts, hidden))
+        self._dense(gates, "gates", torch.float32, (tokens, experts))
+        self._check(self._parts().akv_route(_ptr(x), self._code_of(x), _ptr(router), _ptr(gates), tokens, hidden, experts,
+                                            top, groups, keep, self._stream()), "route")
+
+    def gate_relu_squared(self, up, gates, act) -> None:
+        """act[t, e * ff + j] = gates[t, e] * relu(up[t, e * ff + j])^2 (may be in place)."""
+        tokens, experts = gates.shape
+        self._dense(up, "up")
+        if up.shape[0] != tokens or up.shape[1] % experts:
+            self._refuse(f"up must be [tokens, experts * ff], got {tuple(up.shape)} for {experts} experts")
+        self._dense(act, "act", up.dtype, tuple(up.shape))
+        self._dense(gates, "gates", torch.float32)
+        self._check(self._parts().akv_gate_relu_squared(_ptr(up), _ptr(gates), _ptr(act), self._code_of(up), _long(tokens),
+                                                        experts, up.shape[1] // experts, self._stream()),
+                    "gate_relu_squared")

@@ -1,15 +1,20 @@
-from .base import (CATEGORIES, KernelSet, Norm, PagedKV, Part, Runtime, SlotState, StreamSums, UnnormedRows, build_part,
+from .base import (CATEGORIES, KernelSet, Norm, NormedDelta, PagedKV, Part, Runtime, SlotState, StreamSums, UnnormedRows, build_part,
                    register_part, registered)
-from . import norm, position, linear, feed_forward, attention, block, embedding  # noqa: F401  (registers the kinds)
+from . import (norm, position, linear, feed_forward, attention, block, embedding, latent_attention,  # noqa: F401
+               selective_scan, routed_experts)      # (registers the kinds)
 from .attention import Attention
-from .block import PreNormBlock
-from .embedding import Embedding, LinearHead
+from .block import NoFeedForward, PreNormBlock, SandwichBlock
+from .embedding import Embedding, LinearHead, PairHashEmbedding
 from .feed_forward import SwiGLU
+from .latent_attention import LatentAttention
+from .routed_experts import RoutedExperts
+from .selective_scan import SelectiveScan
 from .linear import Linear
 from .norm import RMSNorm
 from .position import NoPosition, RotaryHalf
 
 __all__ = ["CATEGORIES", "KernelSet", "Norm", "PagedKV", "Part", "Runtime", "SlotState", "StreamSums", "UnnormedRows",
            "build_part", "register_part", "registered",
-           "Attention", "PreNormBlock", "Embedding", "LinearHead", "SwiGLU", "Linear", "RMSNorm", "NoPosition",
+           "NormedDelta", "LatentAttention", "RoutedExperts", "SelectiveScan", "SandwichBlock", "NoFeedForward",
+           "PairHashEmbedding", "Attention", "PreNormBlock", "Embedding", "LinearHead", "SwiGLU", "Linear", "RMSNorm", "NoPosition",
            "RotaryHalf"]

@@ -142,6 +142,8 @@ class Part:
     takes_pending_norm = False
     # (blocks) `pending` may be a `StreamSums`: the residual sum then already holds the branch's output
     takes_stream_sums = False
+    # (blocks) `pending` may be a `NormedDelta`: a branch's output that is still to be normed before it is added
+    takes_normed_delta = False
     # (position encodings) `apply(x, positions, ctx)` instead of `apply(x, positions)`: the encoding reads further
     # integers per token from the step (`ctx.extra`)
     wants_context = False
@@ -185,6 +187,30 @@ class Norm(Part):
         """The float32 vector w of a norm of the form x / rms(x) * w, for a product that leaves rows already
         multiplied by it (`StreamSums.rows`); None for any other norm."""
         return None
+
+    def add_normed(self, stream: torch.Tensor, delta: torch.Tensor) -> None:
+        """stream (float32) += norm(delta), in place."""
+        raise NotImplementedError
+
+    def after(self, stream: torch.Tensor, pending: "NormedDelta | None", out: torch.Tensor) -> torch.Tensor:
+        """stream += pending.norm(pending.delta), if there is one; out = this norm of the new stream - one kernel where
+        the two norms are of a kind that has one."""
+        if pending is not None:
+            pending.settle(stream)
+        return self.forward_residual(stream, None, out)
+
+
+class NormedDelta:
+    """What a block that norms its branches after as well as before hands on as `pending`: the last branch's output
+    `delta` and the norm it has yet to pass before it is added to the residual sum.  A block with
+    `takes_normed_delta = True` does that inside the kernel of its own first norm; for any other reader the model's
+    pass settles it first (`settle`), and the reader sees a residual sum that already holds the branch."""
+
+    def __init__(self, delta: torch.Tensor, norm: "Norm"):
+        self.delta, self.norm = delta, norm
+
+    def settle(self, stream: torch.Tensor) -> None:
+        self.norm.add_normed(stream, self.delta)
 
 
 class StreamSums:

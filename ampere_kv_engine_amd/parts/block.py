@@ -7,7 +7,7 @@ may instead add its output to the stream inside its last product and hand on the
 
 from __future__ import annotations
 
-from .base import Part, build_part, register_part
+from .base import NormedDelta, Part, build_part, register_part
 from .base import StreamSums
 
 
@@ -96,3 +96,64 @@ def _build_prenorm(spec, runtime, mixer=None, feed_forward=None):
 
 
 register_part("block", "prenorm", _build_prenorm)
+
+
+class SandwichBlock(Part):
+    """Every branch is normed before and after:
+        h1 = h + norm_b(mixer(norm_a(h)));  h2 = h1 + norm_d(feed_forward(norm_c(h1)))
+    (a layer without a feed-forward ends after the first line).  The norm after a branch, the addition to the float32
+    residual sum and the norm before the next branch are one kernel (`Norm.after`); the last branch of the block is
+    handed on as a `NormedDelta` and meets the next block's first norm - or the model's end - the same way."""
+    graph_safe = True
+    takes_normed_delta = True
+
+    def __init__(self, spec, runtime, mixer, feed_forward):
+        self.rt = runtime
+        self.hidden = int(spec["hidden_size"])
+        self.mixer, self.feed_forward = mixer, feed_forward
+        self.has_feed_forward = not isinstance(feed_forward, NoFeedForward)
+        names = tuple(spec.get("names", ("norm1", "norm1b", "norm2", "norm2b")))
+        if len(names) != 4:
+            raise ValueError(f"a block of four norms needs four names, got {names}")
+        self.names = names if self.has_feed_forward else names[:2]
+        self.norms = [build_part("norm", spec["norm"], runtime) for _ in self.names]
+
+    def tensors(self, prefix):
+        specs = []
+        for norm, name in zip(self.norms, self.names):
+            specs += norm.tensors(prefix + name)
+        return specs + self.mixer.tensors(prefix) + self.feed_forward.tensors(prefix)
+
+    def load(self, fetch, prefix):
+        for norm, name in zip(self.norms, self.names):
+            norm.load(fetch, prefix + name)
+        self.mixer.load(fetch, prefix)
+        self.feed_forward.load(fetch, prefix)
+
+    def weight_bytes(self):
+        return self.mixer.weight_bytes() + self.feed_forward.weight_bytes() + sum(n.weight_bytes() for n in self.norms)
+
+    def forward(self, stream, pending, ctx, cache, writes_cache=True):
+        if pending is not None and not isinstance(pending, NormedDelta):
+            raise TypeError("a block of four norms is handed a NormedDelta or nothing")
+        ctx.fold_into_stream, ctx.fold_gain = False, None      # no branch of this block adds itself to the stream
+        shape = (stream.shape[0], self.hidden)
+        normed = self.norms[0].after(stream, pending, ctx.arena.take(shape, self.rt.dtype))
+        mixed = NormedDelta(self.mixer.forward(normed, ctx, cache, writes_cache), self.norms[1])
+        if not self.has_feed_forward:
+            return mixed
+        normed = self.norms[2].after(stream, mixed, ctx.arena.take(shape, self.rt.dtype))
+        return NormedDelta(self.feed_forward.forward(normed, ctx), self.norms[3])
+
+
+class NoFeedForward(Part):
+    """The feed-forward of a layer that has none."""
+    graph_safe = True
+
+    def __init__(self, spec=None, runtime=None):
+        pass
+
+
+register_part("block", "sandwich", lambda spec, runtime, mixer=None, feed_forward=None:
+              SandwichBlock(spec, runtime, mixer, feed_forward))
+register_part("feed_forward", "none", NoFeedForward)

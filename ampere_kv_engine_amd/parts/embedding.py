@@ -33,6 +33,32 @@ class Embedding(Part):
         return stream
 
 
+class PairHashEmbedding(Embedding):
+    """The token's row plus a row of a second table that is chosen by the token AND the one before it:
+    row = (previous id * mul_prev + id * mul_cur) mod buckets; a request's first token takes the table's last row
+    (number `buckets`).  The token a request was fed last is part of what it keeps between steps: a word of its slot
+    on the device, so a portion's first token finds its predecessor whatever step brought it."""
+
+    def __init__(self, spec, runtime):
+        super().__init__(spec, runtime)
+        self.pair_name = spec["pair_name"]
+        self.buckets, self.mul_prev, self.mul_cur = int(spec["buckets"]), int(spec["mul_prev"]), int(spec["mul_cur"])
+        if self.buckets <= 0:
+            raise ValueError(f"a table of token pairs needs at least one bucket, got {self.buckets}")
+        self.pairs = None
+
+    def tensors(self, prefix=""):
+        return super().tensors() + [TensorSpec(self.pair_name, (self.buckets + 1, self.hidden), EMBEDDING)]
+
+    def load(self, fetch, prefix=""):
+        super().load(fetch)
+        self.pairs = fetch(self.tensors()[1]).contiguous()
+
+    def forward(self, token_ids, stream, ctx=None):
+        self.rt.kernels.embed_pairs(token_ids, self.weight, self.pairs, self.buckets, self.mul_prev, self.mul_cur, stream, ctx)
+        return stream
+
+
 class LinearHead(Part):
     """logits = x W^T in float32.  When `tied_to` names the embedding, the head uses that matrix and the
     file may leave the head's own tensor out."""
@@ -64,4 +90,5 @@ class LinearHead(Part):
 
 
 register_part("embedding", "embedding", Embedding)
+register_part("embedding", "pair_hash_embedding", PairHashEmbedding)
 register_part("head", "linear_head", LinearHead)

@@ -1,6 +1,11 @@
 """RMSNorm (ampere_kv/runner.py:48-57): x * rsqrt(mean(x^2) + eps), rounded to the activation dtype, then
 times the weight.  Statistics are formed in float32.  The weight is kept in float32 (a widening of what the
-file stores, so the product equals the reference's)."""
+file stores, so the product equals the reference's).
+
+With `single_rounding` the norm is float32 from the statistics to the product with the weight, and a result is
+rounded once, when it is stored (designs that say their norms are computed in 32-bit).  Such a norm takes no part in
+the folding of norms into products; it can be added to the residual sum as it is computed (`add_normed`) and chained
+with the norm that follows (`after`): the norm kernel of blocks that norm a branch before and after."""
 
 from __future__ import annotations
 
@@ -14,6 +19,7 @@ class RMSNorm(Norm):
     def __init__(self, spec, runtime):
         self.size = int(spec["size"])
         self.eps = float(spec["eps"])
+        self.single_rounding = bool(spec.get("single_rounding", False))
         self.rt = runtime
         self.weight: torch.Tensor | None = None
 
@@ -28,26 +34,45 @@ class RMSNorm(Norm):
 
     def forward(self, x: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
         """x [..., size] in the activation dtype -> out of the same shape."""
+        if self.single_rounding:
+            raise NotImplementedError("a norm with one rounding reads the float32 residual sum (forward_residual, after)")
         self.rt.kernels.rmsnorm(x.view(-1, self.size), self.weight, self.eps, out.view(-1, self.size))
         return out
 
     def forward_residual(self, stream: torch.Tensor, delta: torch.Tensor | None, out: torch.Tensor) -> torch.Tensor:
         """stream [tokens, size] float32 is the residual sum; `delta` (activation dtype) is added to it in
         float32 first, then the sum is normed into `out` (activation dtype)."""
+        if self.single_rounding:
+            self.rt.kernels.norm_add_norm(stream, delta, None, 0.0, self.weight, self.eps, out)
+            return out
         self.rt.kernels.add_rmsnorm(stream, delta, self.weight, self.eps, out)
         return out
 
+    def add_normed(self, stream: torch.Tensor, delta: torch.Tensor) -> None:
+        if not self.single_rounding:
+            raise NotImplementedError("only a norm with one rounding is added to the residual sum as it is computed")
+        self.rt.kernels.norm_add_norm(stream, delta, self.weight, self.eps, None, 0.0, None)
+
+    def after(self, stream, pending, out):
+        if pending is None or not (self.single_rounding and type(pending.norm) is RMSNorm and pending.norm.single_rounding):
+            return super().after(stream, pending, out)
+        self.rt.kernels.norm_add_norm(stream, pending.delta, pending.norm.weight, pending.norm.eps, self.weight, self.eps, out)
+        return out
 
     def pending(self, stream: torch.Tensor, delta: torch.Tensor | None, stream_out: torch.Tensor, arena) -> "PendingNorm":
         """`forward_residual` not yet computed: for a consumer whose first product can compute it itself."""
+        if self.single_rounding:
+            return None
         return PendingNorm(self, stream, delta, stream_out, arena)
 
     def fold_gain(self):
-        return self.weight
+        return None if self.single_rounding else self.weight
 
     def scaled(self, stream: torch.Tensor, sums: "StreamSums", arena) -> "ScaledNorm":
         """The norm of a residual sum whose rows' sums of squares are already known (`StreamSums`): for a consumer
         whose first product can norm its rows itself from them."""
+        if self.single_rounding:
+            return None
         return ScaledNorm(self, stream, sums, arena)
 
 

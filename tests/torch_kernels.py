@@ -250,6 +250,122 @@ class TorchKernels(KernelSet):
                 merged[:, head] = scores.softmax(-1) @ values[:, head // group]
             out[first:last] = merged.reshape(last - first, q_heads * head_dim).to(out.dtype)
 
+    # ---- designs with float32 norms: pair embedding, norm before and after, latent attention, scan, routing ------------
+    def embed_pairs(self, ids, table, pairs, buckets, mul_prev, mul_cur, out, ctx):
+        """out[n] = table[id] + pairs[row]; row = (previous * mul_prev + id * mul_cur) mod buckets, `buckets` at position
+        0; the previous id of a portion's first token is word 7 of the request's slot, which then takes the portion's
+        last id."""
+        words = ctx.slot_words
+        slots = ctx.seq_slots.long()[ctx.seq_of_token.long()]
+        cur = ids.long().clone()
+        cur = torch.where(cur == -1, words[slots, 1].long(), cur)
+        prev = torch.roll(cur, 1)
+        starts = ctx.q_start.long()[:-1]
+        prev[starts] = words[ctx.seq_slots.long(), 7].long()
+        rows = (prev * mul_prev + cur * mul_cur) % buckets
+        rows = torch.where(ctx.positions.long() == 0, torch.full_like(rows, buckets), rows)
+        out.copy_(table[cur].float() + pairs[rows].float())
+        words[ctx.seq_slots.long(), 7] = cur[ctx.q_start.long()[1:] - 1].int()
+
+    def norm_add_norm(self, stream, delta, post_weight, post_eps, pre_weight, pre_eps, out):
+        if delta is not None:
+            d = delta.float()
+            if post_weight is not None:
+                d = d * torch.rsqrt((d * d).mean(-1, keepdim=True) + post_eps) * post_weight
+            stream += d
+        if out is not None:
+            out.copy_((stream * torch.rsqrt((stream * stream).mean(-1, keepdim=True) + pre_eps) * pre_weight).to(out.dtype))
+
+    @staticmethod
+    def _turn(x, positions, table, rot_dims):
+        """x [..., tokens, heads, rot] float: the first rot_dims dimensions rotated in halves by the table's angles."""
+        half = rot_dims // 2
+        cos = table[positions.long(), :, 0][:, None, :]
+        sin = table[positions.long(), :, 1][:, None, :]
+        u, v = x[..., :half], x[..., half:rot_dims]
+        return torch.cat((u * cos - v * sin, v * cos + u * sin, x[..., rot_dims:]), dim=-1)
+
+    def latent_encode(self, down, q_rank, kv_rank, rot, rot_dims, q_weight, kv_weight, eps, table, positions, slot_map,
+                      cq, records):
+        d = down.float()
+        ql = d[:, :q_rank]
+        cq.copy_((ql * torch.rsqrt((ql * ql).mean(-1, keepdim=True) + eps) * q_weight).to(cq.dtype))
+        if records is None:
+            return
+        c = d[:, q_rank:q_rank + kv_rank]
+        c = c * torch.rsqrt((c * c).mean(-1, keepdim=True) + eps) * kv_weight
+        key = self._turn(d[:, None, q_rank + kv_rank:], positions, table, rot_dims)[:, 0]
+        flat = records.view(-1, kv_rank + rot)
+        flat[slot_map.long()] = torch.cat((c, key), dim=-1).to(records.dtype)
+
+    def rotate_queries(self, q, heads, dim, rot, rot_dims, table, positions, q_abs, at):
+        part = q.float().view(q.shape[0], heads, dim + rot)[..., dim:]
+        q_abs[..., at:at + rot] = self._turn(part, positions, table, rot_dims)
+
+    def heads_linear(self, x, x_width, weight, y, y_width):
+        heads, ins, outs = weight.shape
+        y[..., :outs] = torch.einsum("thi,hio->tho", x[..., :ins].float(), weight.float()).to(y.dtype)
+
+    def latent_attend(self, q_abs, records, ctx, meta, heads, kv_rank, scale, window, out):
+        page_size = records.shape[2]
+        table = meta.block_table.cpu()
+        if getattr(meta, "rows", None) is not None:
+            table = table[meta.rows.cpu().long()]
+        positions = ctx.positions.cpu().long()
+        for r in range(ctx.num_seqs):
+            first, last = ctx.host_q_start[r], ctx.host_q_start[r + 1]
+            for n in range(first, last):
+                pos = int(positions[n])
+                lowest = 0 if window is None else max(0, pos - window + 1)
+                key_pos = torch.arange(lowest, pos + 1)
+                pages = table[r][key_pos // page_size].long()
+                assert (pages >= 0).all(), "attention would read a page that was given back"
+                recs = records[pages, 0, key_pos % page_size].float()           # [S, width]
+                weights = ((q_abs[n] @ recs.T) * scale).softmax(-1)             # [heads, S]
+                out[n] = weights @ recs[:, :kv_rank]
+
+    def conv_silu(self, xz, channels, weight, bias, state, n_state, ctx, out):
+        taps = weight.shape[1]
+        conv_at = channels * n_state
+        for r in range(ctx.num_seqs):
+            first, last, slot = ctx.host_q_start[r], ctx.host_q_start[r + 1], ctx.host_seq_slots[r]
+            kept = state[slot, conv_at:].view(taps - 1, channels)
+            seen = torch.cat((kept, xz[first:last, :channels].float()), dim=0)
+            for t in range(last - first):
+                acc = (seen[t:t + taps] * weight.float().T).sum(0) + bias.float()
+                out[first + t] = (acc * torch.sigmoid(acc)).to(out.dtype)
+            state[slot, conv_at:] = seen[seen.shape[0] - (taps - 1):].reshape(-1)
+
+    def selective_scan(self, x, dt, bc, xz, a, d, state, taps, ctx, out):
+        channels, n_state = a.shape
+        for r in range(ctx.num_seqs):
+            first, last, slot = ctx.host_q_start[r], ctx.host_q_start[r + 1], ctx.host_seq_slots[r]
+            S = state[slot, :channels * n_state].view(channels, n_state).clone()
+            for t in range(first, last):
+                step = torch.nn.functional.softplus(dt[t], threshold=20.0)
+                xv = x[t].float()
+                S = torch.exp(step[:, None] * a) * S + (step * xv)[:, None] * bc[t, None, :n_state]
+                y = S @ bc[t, n_state:] + d * xv
+                z = xz[t, channels:].float()
+                out[t] = (y * z * torch.sigmoid(z)).to(out.dtype)
+            state[slot, :channels * n_state] = S.reshape(-1)
+
+    def route(self, x, router, gates, top, groups, keep):
+        scores = (x.float() @ router.T).softmax(-1)
+        tokens, experts = scores.shape
+        best = scores.view(tokens, groups, experts // groups).amax(-1)
+        allowed = torch.zeros(tokens, groups, dtype=torch.bool)
+        allowed.scatter_(1, best.topk(keep, dim=-1).indices, True)
+        allowed = allowed[:, :, None].expand(tokens, groups, experts // groups).reshape(tokens, experts)
+        chosen = scores.masked_fill(~allowed, -1.0).topk(top, dim=-1).indices
+        gates.zero_()
+        gates.scatter_(1, chosen, scores.gather(1, chosen))
+
+    def gate_relu_squared(self, up, gates, act):
+        tokens, experts = gates.shape
+        u = torch.relu(up.float()).view(tokens, experts, -1) ** 2
+        act.copy_((u * gates[:, :, None]).view(tokens, -1).to(act.dtype))
+
     # ---- sampling -----------------------------------------------------------------------------------------
     def sample(self, logits, temperature, seeds, draws, out):
         """temperature 0: the largest logit, ties to the lowest id.  Otherwise the Gumbel-max draw
