@@ -187,3 +187,17 @@ def forward(config: dict, weights: dict, ids: list[int], return_layers: bool = F
         after.append(x.clone())
     logits = rms_norm(x, w["final.norm"], eps) @ w["head"].T
     return (logits, torch.stack(after)) if return_layers else logits
+
+
+def attend_records(q_abs: torch.Tensor, records: torch.Tensor, positions: list[int], window: int | None, scale: float,
+                   kv_rank: int) -> torch.Tensor:
+    """The attention in its absorbed form, for checks of that step alone: query n [heads, width] at `positions[n]`
+    attends the records [length, width] of positions within its window; the values are the records' first kv_rank
+    dimensions.  -> [n, heads, kv_rank]"""
+    out = torch.zeros(q_abs.shape[0], q_abs.shape[1], kv_rank)
+    for n, pos in enumerate(positions):
+        lo = 0 if window is None else max(0, pos - window + 1)
+        seen = records[lo:pos + 1]
+        p = torch.softmax((q_abs[n] @ seen.T) * scale, dim=-1)
+        out[n] = p @ seen[:, :kv_rank]
+    return out
