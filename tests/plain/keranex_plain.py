@@ -8,8 +8,6 @@ Notation: n tokens, d model width, H heads.  Linear weights are [out, in] and ap
 
 from __future__ import annotations
 
-import math
-
 import torch
 
 
@@ -17,10 +15,6 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor | None, eps: float) -> torch.
     """x / sqrt(mean(x^2) + eps) [* weight], over the last axis."""
     y = x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps)
     return y if weight is None else y * weight
-
-
-def gelu_tanh(z: torch.Tensor) -> torch.Tensor:
-    return 0.5 * z * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z ** 3)))
 
 
 def silu(z: torch.Tensor) -> torch.Tensor:

@@ -294,7 +294,7 @@ def test_one_key_stands_out_just_inside_and_just_outside_the_window(hip, window,
             want = plain.attend_records(q_abs, boosted, list(range(history, history + count)), window, 1.0, kv_rank)
             torch.testing.assert_close(out.cpu(), want, rtol=1e-4, atol=1e-4)
             dominated = torch.allclose(out[-1, 0].cpu(), boosted[at, :kv_rank], rtol=1e-2, atol=1e-2)
-            assert dominated == (seen and window > 1 or offset == 0), (offset, seen)
+            assert dominated == seen, (offset, seen)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
