@@ -1,0 +1,119 @@
+"""Prefill and decode throughput of the Keranex design at sizes that resemble a real model's layers (random weights),
+beside the dense Qwen3 decoder at equal width, depth, heads and active feed-forward width - the closest model the
+engine has.  `python bench.py --workload keranex [--design-sizes s,m] [--layers L]` prints one JSON line per size:
+
+  prefill  one request's 2,048-token prompt fed whole: tokens per second and milliseconds
+  decode   `batch` requests with caches of `context` tokens, one token each per step, chosen greedily: tokens per second
+
+A Keranex model here repeats the pattern [attention over a latent, the same, selective scan, attention reading the
+second layer's latent], every layer with a routed feed-forward; its Qwen3 neighbour has as many layers of grouped-query
+attention (a quarter as many kv heads) and a dense feed-forward as wide as the experts a token uses.
+"""
+
+from __future__ import annotations
+
+import json
+import time
+
+PAGE_SIZE, PREFILL_TOKENS = 16, 2048
+
+SIZES = {
+    "s": dict(width=2048, vocab=32768, heads=16, dim=128, rot=64, vdim=128, kv_rank=512, q_rank=768, window=1024,
+              inner=4096, state=16, dt_rank=128, conv=4, experts=16, top=2, groups=4, keep=2, ff=1024),
+    "m": dict(width=4096, vocab=65536, heads=32, dim=128, rot=64, vdim=128, kv_rank=512, q_rank=1536, window=2048,
+              inner=8192, state=16, dt_rank=256, conv=4, experts=32, top=4, groups=8, keep=4, ff=1024),
+}
+
+
+def keranex_config(size: dict, layers: int) -> dict:
+    latent = lambda **more: dict(heads=size["heads"], dim=size["dim"], rot_dim=size["rot"], vdim=size["vdim"],
+                                 kv_rank=size["kv_rank"], q_rank=size["q_rank"], mask=dict(size=size["window"]),
+                                 scale=(size["dim"] + size["rot"]) ** -0.5, rot=dict(base=10000.0, dims=size["rot"]), **more)
+    mlp = dict(kind="moe", expert=dict(ff=size["ff"]), router=dict(experts=size["experts"], top=size["top"],
+               groups=dict(count=size["groups"], keep=size["keep"])))
+    out = []
+    for index in range(layers):
+        place = index % 4
+        if place == 2:
+            out.append(dict(type="mamba1", mixer=dict(inner=size["inner"], state=size["state"], dt_rank=size["dt_rank"],
+                                                      conv=size["conv"]), mlp=mlp))
+        elif place == 3:
+            out.append(dict(type="latent_attention", mixer=latent(kv_from=index - 2), mlp=mlp))
+        else:
+            out.append(dict(type="latent_attention", mixer=latent(), mlp=mlp))
+    return dict(architecture="Keranex", vocab=size["vocab"], width=size["width"], norm=dict(eps=1e-5),
+                embedding=dict(bigram=dict(buckets=size["vocab"] - 1, mul_prev=127, mul_cur=17)), layers=out)
+
+
+def qwen3_config(size: dict, layers: int) -> dict:
+    return dict(architectures=["Qwen3ForCausalLM"], num_hidden_layers=layers, hidden_size=size["width"],
+                num_attention_heads=size["heads"], num_key_value_heads=max(size["heads"] // 4, 1), head_dim=128,
+                intermediate_size=size["top"] * size["ff"], vocab_size=size["vocab"], rope_theta=1000000.0,
+                rms_norm_eps=1e-6, tie_word_embeddings=False, hidden_act="silu")
+
+
+def measure(config, batch: int, context: int, steps: int, warmup: int, graphs: bool = True) -> dict:
+    import torch
+    from .config import EngineConfig
+    from .engine import LAST_TOKEN, Engine, StepEntry
+    per_request = context + warmup + steps + 8
+    pages = batch * ((per_request + PAGE_SIZE - 1) // PAGE_SIZE + 1) + PREFILL_TOKENS // PAGE_SIZE + 2
+    engine = Engine.from_random(config, seed=0, engine_config=EngineConfig(
+        dtype="bfloat16", page_size=PAGE_SIZE, num_pages=pages, max_seqs=batch + 1, max_batched_tokens=PREFILL_TOKENS,
+        max_seq_len=max(per_request, PREFILL_TOKENS) + PAGE_SIZE, device="cuda:0", decode_graphs=graphs))
+    for group in engine.cache.groups:       # any finite records: what they hold does not change the time
+        group.pages.normal_(0.0, 0.5)
+    generator = torch.Generator().manual_seed(0)
+    sync = lambda: torch.cuda.synchronize(engine.device)
+    vocab = engine.spec.vocab_size
+    # ---- prefill
+    samples = []
+    for run in range(4):
+        ids = torch.randint(0, vocab, (PREFILL_TOKENS,), generator=generator).tolist()
+        seq = engine.open(f"p{run}")
+        sync()
+        started = time.perf_counter()
+        engine.step([StepEntry(seq, ids, [PREFILL_TOKENS - 1])])
+        sync()
+        samples.append(time.perf_counter() - started)
+        engine.close(seq)
+    prefill = sorted(samples[1:])[1]
+    # ---- decode
+    seqs = [engine.open(f"d{i}") for i in range(batch)]
+    for seq in seqs:
+        engine.cache.reserve(seq, context - 1)
+    first = torch.randint(0, vocab, (batch,), generator=generator).tolist()
+    engine.choose(engine.step([StepEntry(seq, [token], [0]) for seq, token in zip(seqs, first)], borrow_logits=True))
+    for _ in range(3 + warmup):
+        engine.choose(engine.step([StepEntry(seq, LAST_TOKEN, [0]) for seq in seqs], borrow_logits=True))
+    sync()
+    started = time.perf_counter()
+    for _ in range(steps):
+        engine.choose(engine.step([StepEntry(seq, LAST_TOKEN, [0]) for seq in seqs], borrow_logits=True))
+    sync()
+    decode = (time.perf_counter() - started) / steps
+    for seq in seqs:
+        engine.close(seq)
+    out = dict(prefill_tok_per_s=round(PREFILL_TOKENS / prefill, 1), prefill_ms=round(prefill * 1000, 3),
+               decode_tok_per_s=round(batch / decode, 1), decode_ms_per_step=round(decode * 1000, 3),
+               weight_gb_per_step=round(engine.model.weight_bytes_per_step() / 1e9, 3))
+    del engine
+    torch.cuda.empty_cache()
+    return out
+
+
+def design_workload(sizes: str, layers: int | None, batch: int, context: int, steps: int, warmup: int,
+                    graphs: bool = True, only: str = "") -> int:
+    from .config import KeranexConfig, Qwen3Config
+    for name in [s for s in sizes.split(",") if s]:
+        size = SIZES[name]
+        count = layers or 8
+        line = {"workload": "keranex", "sizes": name, "layers": count, "batch": batch, "context": context,
+                "prefill_tokens": PREFILL_TOKENS, "dtype": "bf16", "data": "synthetic: random-init weights, random token ids",
+                "shape": size}
+        if only in ("", "keranex"):
+            line["keranex"] = measure(KeranexConfig.from_dict(keranex_config(size, count)), batch, context, steps, warmup, graphs)
+        if only in ("", "qwen3"):
+            line["qwen3_equal_size"] = measure(Qwen3Config.from_dict(qwen3_config(size, count)), batch, context, steps, warmup, graphs)
+        print(json.dumps(line), flush=True)
+    return 0

@@ -43,6 +43,14 @@ int akv_latent_attend(const float* q_abs, const void* records, int dtype, const 
                       const int* block_table, const int* table_rows, int table_width, float* out, int tokens, int heads,
                       int kv_rank, int width, int page_size, long num_pages, float scale, int window,
                       hipStream_t stream);
+// The same on the matrix cores, for bfloat16, heads that are a multiple of 16, records a multiple of 32 wide, latents
+// of 128, 256 or 512 and pages of a multiple of 8 tokens (-2 otherwise).  `latents_t` [pages, kv_rank, page]: the
+// records' first kv_rank dimensions once more, keys contiguous.  q_abs [tokens, heads, width] and out [tokens, heads,
+// kv_rank] are bfloat16.
+int akv_latent_attend_mfma(const void* q_abs, const void* records, const void* latents_t, const int* seq_of_token,
+                           const int* positions, const int* block_table, const int* table_rows, int table_width,
+                           void* out, int tokens, int heads, int kv_rank, int width, int page_size, long num_pages,
+                           float scale, int window, hipStream_t stream);
 
 // ---- selective scan (selective_scan.hip) ----------------------------------------------------------------------------
 // x [tokens, channels] at `x_stride` per token; state [slots, state_stride] float32 holds (taps - 1) x channels at

@@ -9,6 +9,7 @@
 // scores, softmax and the weighted sums are float32.
 
 #include "common.h"
+#include "mfma_tiles.h"
 #include "api_parts.h"
 
 using namespace akv;
@@ -248,6 +249,173 @@ __global__ __launch_bounds__(512) void latent_attend_kernel(
   }
 }
 
+
+// ---- the same on the matrix cores (bfloat16) --------------------------------------------------------------------------
+// For layers whose heads are a multiple of 16: a wave is one token and 16 of its heads - the 16 columns of the matrix
+// instruction, which all see the same keys.  S^T = K Q^T (keys are the A operand, 16 bytes a lane straight from the
+// records) and O^T = C^T P^T, where C^T, the latents with the keys contiguous, is a second copy that the layer keeps
+// beside the records as [kv_rank, page] per page: 8 keys of a dimension are then one 16-byte load, and the weights
+// are the B operand as they stand in the registers.  Row rho of a score tile is key base + (rho / 4) * 8 + j * 4 +
+// rho % 4 (j: which of a step's two tiles), so that a lane's 8 weights of a step are 8 consecutive keys.  Weights
+// enter the second product as high + low bfloat16.  Steps of 32 keys lie at absolute positions.
+typedef __attribute__((ext_vector_type(2))) float floatx2;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+
+template <int VT>      // kv_rank / 16
+__global__ __launch_bounds__(256) void latent_attend_mfma_kernel(
+    const bf16_t* __restrict__ q_abs, const bf16_t* __restrict__ records, const bf16_t* __restrict__ latents_t,
+    const int* __restrict__ seq_of_token, const int* __restrict__ positions, const int* __restrict__ block_table,
+    const int* __restrict__ table_rows, int table_width, bf16_t* __restrict__ out, long tiles, int heads, int width,
+    int page_size, long num_pages, float scale_log2, int window) {
+  extern __shared__ unsigned char lds_bytes[];
+  constexpr int kv_rank = VT * 16;
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
+  const long tile = static_cast<long>(blockIdx.x) * (blockDim.x / kWave) + wave;
+  if (tile >= tiles) return;
+  const int rho = lane & 15, g = lane >> 4;
+  const long n = tile * 16 / heads;                         // the tile's token (heads are a multiple of 16)
+  const int r = table_rows != nullptr ? table_rows[seq_of_token[n]] : seq_of_token[n];
+  const int pos = positions[n];
+  const int lowest = window > 0 ? max(0, pos - window + 1) : 0;
+  const int* table = block_table + static_cast<long>(r) * table_width;
+  // the tile's 16 query rows into LDS, rows 16 bytes further apart than they are wide
+  const int chunks = width / 8, stride = (chunks + 1) * 16;
+  unsigned char* qs = lds_bytes + static_cast<size_t>(wave) * 16 * stride;
+  const uintx4* q_rows = reinterpret_cast<const uintx4*>(q_abs + tile * 16 * width);
+  for (int e = lane; e < 16 * chunks; e += kWave)
+    *reinterpret_cast<uintx4*>(qs + (e / chunks) * stride + (e % chunks) * 16) = q_rows[e];
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  const unsigned char* q_mine = qs + rho * stride + g * 16;
+
+  // the token's own slot: always written, what a lane reads in place of a key it may not see
+  const long own_page = table[pos / page_size];
+  const bool lost = own_page < 0 || own_page >= num_pages;
+  const long safe_page = lost ? 0 : own_page;
+  const long safe_slot = safe_page * page_size + pos % page_size;
+
+  floatx4 o[VT];
+#pragma unroll
+  for (int dt = 0; dt < VT; ++dt) o[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+  bool poisoned = lost;
+  const int steps32 = width / 32;
+
+  for (int base = lowest & ~31; base <= pos; base += 32) {
+    const bool edge = base < lowest || base + 31 > pos;
+    // ---- scores: two tiles of 16 keys ---------------------------------------------------------------------------
+    floatx4 s[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int key = base + (rho >> 2) * 8 + j * 4 + (rho & 3);
+      long slot = safe_slot;
+      if (key >= lowest && key <= pos) {
+        const long page = table[key / page_size];
+        if (page < 0 || page >= num_pages) poisoned = true;
+        else slot = page * page_size + key % page_size;
+      }
+      const uintx4* row = reinterpret_cast<const uintx4*>(records + slot * width) + g;
+      floatx4 acc = floatx4{0.f, 0.f, 0.f, 0.f};
+      for (int t = 0; t < steps32; ++t)
+        acc = mfma16(row[t * 4], *reinterpret_cast<const uintx4*>(q_mine + t * 64), acc);
+      s[j] = acc;
+    }
+    if (edge) {
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int key = base + g * 8 + j * 4 + i;
+          if (key < lowest || key > pos) s[j][i] = -INFINITY;
+        }
+    }
+    float top = fmaxf(fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3])),
+                      fmaxf(fmaxf(s[1][0], s[1][1]), fmaxf(s[1][2], s[1][3])));
+    top = fmaxf(top, __shfl_xor(top, 16, kWave));
+    top = fmaxf(top, __shfl_xor(top, 32, kWave));
+    const float m_new = fmaxf(m, top * scale_log2);
+    const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+    const float correction = __builtin_amdgcn_exp2f(m - m_safe);
+    floatx2 p[4];
+    float sum = 0.f;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      p[e][0] = __builtin_amdgcn_exp2f(fmaf(s[e >> 1][(e & 1) * 2], scale_log2, -m_safe));
+      p[e][1] = __builtin_amdgcn_exp2f(fmaf(s[e >> 1][(e & 1) * 2 + 1], scale_log2, -m_safe));
+      sum += p[e][0] + p[e][1];
+    }
+    l = l * correction + sum;
+    m = m_new;
+    uint32_t high[4], low[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      high[e] = __builtin_bit_cast(uint32_t, __builtin_convertvector(p[e], bf16x2));
+      const floatx2 rest = {p[e][0] - __uint_as_float(high[e] << 16), p[e][1] - __uint_as_float(high[e] & 0xffff0000u)};
+      low[e] = __builtin_bit_cast(uint32_t, __builtin_convertvector(rest, bf16x2));
+    }
+    const uintx4 p_high = uintx4{high[0], high[1], high[2], high[3]}, p_low = uintx4{low[0], low[1], low[2], low[3]};
+    if (__any(correction != 1.f)) {
+#pragma unroll
+      for (int dt = 0; dt < VT; ++dt) o[dt] *= correction;
+    }
+    // ---- O^T += C^T P^T: this lane's 8 keys base + g * 8 .. + 7 of dimension dt * 16 + rho ---------------------------
+    const int first_key = base + g * 8;
+    long value_page = safe_page;
+    int value_at = 0;
+    uint32_t keep[4] = {0u, 0u, 0u, 0u};          // which of the 8 keys count (others may hold anything)
+    if (first_key + 7 >= lowest && first_key <= pos) {
+      const long page = table[first_key / page_size];
+      if (page >= 0 && page < num_pages) {
+        value_page = page;
+        value_at = first_key % page_size;
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (first_key + e >= lowest && first_key + e <= pos) keep[e >> 1] |= (e & 1) ? 0xffff0000u : 0x0000ffffu;
+      } else {
+        poisoned = true;
+      }
+    }
+    const bf16_t* values = latents_t + (value_page * kv_rank + rho) * page_size + value_at;
+#pragma unroll
+    for (int dt = 0; dt < VT; ++dt) {
+      uintx4 v = *reinterpret_cast<const uintx4*>(values + static_cast<long>(dt) * 16 * page_size);
+      if (edge) v = uintx4{v[0] & keep[0], v[1] & keep[1], v[2] & keep[2], v[3] & keep[3]};
+      o[dt] = mfma16(v, p_low, mfma16(v, p_high, o[dt]));
+    }
+  }
+  l += __shfl_xor(l, 16, kWave);
+  l += __shfl_xor(l, 32, kWave);
+  const bool any_poison = __any(poisoned);
+  const float inverse = 1.f / l;
+  bf16_t* dst = out + (tile * 16 + rho) * kv_rank + g * 4;
+#pragma unroll
+  for (int dt = 0; dt < VT; ++dt) {
+    floatx4 v = o[dt] * inverse;
+    if (any_poison) v = floatx4{__uint_as_float(kPoison), __uint_as_float(kPoison), __uint_as_float(kPoison), __uint_as_float(kPoison)};
+    store4<bf16_t>(dst + dt * 16, v);
+  }
+}
+
+template <int VT>
+int launch_attend_mfma(const void* q_abs, const void* records, const void* latents_t, const int* seq_of_token,
+                       const int* positions, const int* block_table, const int* table_rows, int table_width, void* out,
+                       long tiles, int heads, int width, int page_size, long num_pages, float scale, int window,
+                       hipStream_t stream) {
+  constexpr int waves = 4;
+  const size_t lds = static_cast<size_t>(waves) * 16 * (width / 8 + 1) * 16;
+  auto kernel = latent_attend_mfma_kernel<VT>;
+  if (lds > device_facts().lds_bytes) return -2;
+  if (lds > 64 * 1024 && hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                             static_cast<int>(lds)) != hipSuccess)
+    return -2;
+  kernel<<<static_cast<unsigned>((tiles + waves - 1) / waves), waves * kWave, lds, stream>>>(
+      static_cast<const bf16_t*>(q_abs), static_cast<const bf16_t*>(records), static_cast<const bf16_t*>(latents_t),
+      seq_of_token, positions, block_table, table_rows, table_width, static_cast<bf16_t*>(out), tiles, heads, width,
+      page_size, num_pages, scale * 1.4426950408889634f, window);
+  return AKV_LAUNCH_STATUS();
+}
+
 template <typename T, int KT>
 int launch_attend(const float* q_abs, const void* records, const int* seq_of_token, const int* positions,
                   const int* block_table, const int* table_rows, int table_width, float* out, int tokens, int heads,
@@ -344,6 +512,23 @@ int akv_latent_attend(const float* q_abs, const void* records, int dtype, const 
     AKV_ATTEND(T, 8);
   });
 #undef AKV_ATTEND
+  return -2;
+}
+
+int akv_latent_attend_mfma(const void* q_abs, const void* records, const void* latents_t, const int* seq_of_token,
+                           const int* positions, const int* block_table, const int* table_rows, int table_width,
+                           void* out, int tokens, int heads, int kv_rank, int width, int page_size, long num_pages,
+                           float scale, int window, hipStream_t stream) {
+  if (tokens <= 0) return 0;
+  if (heads % 16 || width % 32 || kv_rank % 16 || kv_rank > width || page_size % 8) return -2;
+  const long tiles = static_cast<long>(tokens) * heads / 16;
+#define AKV_MFMA(VT)                                                                                                   \
+  return launch_attend_mfma<VT>(q_abs, records, latents_t, seq_of_token, positions, block_table, table_rows, table_width, \
+                                out, tiles, heads, width, page_size, num_pages, scale, window, stream)
+  if (kv_rank == 128) AKV_MFMA(8);
+  if (kv_rank == 256) AKV_MFMA(16);
+  if (kv_rank == 512) AKV_MFMA(32);
+#undef AKV_MFMA
   return -2;
 }
 }
