@@ -123,9 +123,12 @@ class KeranexConfig:
     # ---- the model this configuration describes -------------------------------------------------------
     def cache_window(self, owner: int) -> int:
         """Tokens that the layer which owns a latent cache must keep: the widest window among the layers that read it."""
-        sizes = [layer["mixer"]["mask"]["size"] for index, layer in enumerate(self.layers)
-                 if layer["type"] == "latent_attention" and (index == owner or layer["mixer"].get("kv_from") == owner)]
-        return max(sizes)
+        return max(self.layers[index]["mixer"]["mask"]["size"] for index in self.cache_readers(owner))
+
+    def cache_readers(self, owner: int) -> list[int]:
+        """The layers that read the records of layer `owner`: itself and those that name it as `kv_from`."""
+        return [index for index, layer in enumerate(self.layers)
+                if layer["type"] == "latent_attention" and (index == owner or layer["mixer"].get("kv_from") == owner)]
 
     def to_model_spec(self) -> ModelSpec:
         raw = self.raw
@@ -141,7 +144,8 @@ class KeranexConfig:
                              rotated_dim=m["rot_dim"], value_dim=m["vdim"], kv_rank=m["kv_rank"], q_rank=m["q_rank"],
                              scale=float(m["scale"]), window=m["mask"]["size"], cache_window=self.cache_window(owner),
                              rotary_dims=m["rot"]["dims"], rotary_base=float(m["rot"]["base"]), eps=eps,
-                             own_latent=source is None, name="mix")
+                             own_latent=source is None, name="mix",
+                             reader_heads=tuple(self.layers[r]["mixer"]["heads"] for r in self.cache_readers(owner)))
                 order.append(RunEntry(index, owner, writes_cache=source is None))
             else:
                 mixer = part("selective_scan", hidden_size=hidden, inner=m["inner"], state=m["state"],

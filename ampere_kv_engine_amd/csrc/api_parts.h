@@ -25,15 +25,16 @@ int akv_norm_add_norm(float* stream_buf, const void* delta, const float* post_we
 
 // ---- attention over a compressed latent (latent_attention.hip) ------------------------------------------------------
 // down [tokens, q_rank (+ kv_rank + rot)]: q latent normed into `cq`; with `records`: the kv latent normed and the
-// shared key part rotated (first `rot_dims` of its `rot` dimensions) into the token's record [kv_rank + rot].
+// shared key part rotated (first `rot_dims` of its `rot` dimensions) into the token's record [kv_rank + rot].  With
+// `latents_t` [pages, kv_rank, page_size] the normed latent is written there too, keys contiguous.
 int akv_latent_encode(const void* down, int dtype, int tokens, int q_rank, int kv_rank, int rot, int rot_dims,
                       const float* q_weight, const float* kv_weight, float eps, const float* table, int table_positions,
                       const int* positions, const int* slot_map, void* cq, void* records, long record_slots,
-                      hipStream_t stream);
-// q [tokens, heads, dim + rot] -> q_abs[..., at : at + rot] (float32, row width `width`), rotated by position
+                      void* latents_t, int page_size, hipStream_t stream);
+// q [tokens, heads, dim + rot] -> q_abs[..., at : at + rot] (float32 or bfloat16, row width `width`), rotated by position
 int akv_rotate_queries(const void* q, int dtype, long tokens, int heads, int dim, int rot, int rot_dims,
-                       const float* table, int table_positions, const int* positions, float* q_abs, int width, int at,
-                       hipStream_t stream);
+                       const float* table, int table_positions, const int* positions, void* q_abs, int out_dtype,
+                       int width, int at, hipStream_t stream);
 // y[t, h, j] = sum_i x[t, h, i] * w[h, i, j]   (w [heads, ins, outs]; x and y addressed by token and head strides)
 int akv_heads_linear(const void* x, int x_dtype, long x_token_stride, long x_head_stride, const void* w, int w_dtype,
                      void* y, int y_dtype, long y_token_stride, long y_head_stride, int tokens, int heads, int ins,

@@ -25,7 +25,7 @@ __global__ __launch_bounds__(256) void latent_encode_kernel(
     const T* __restrict__ down, int q_rank, int kv_rank, int rot, int rot_dims, const float* __restrict__ q_weight,
     const float* __restrict__ kv_weight, float eps, const float* __restrict__ table, int table_positions,
     const int* __restrict__ positions, const int* __restrict__ slot_map, T* __restrict__ cq, T* __restrict__ records,
-    long record_slots) {
+    long record_slots, T* __restrict__ latents_t, int page_size) {
   __shared__ float scratch[16];
   const int n = blockIdx.x;
   const bool writes = records != nullptr;
@@ -50,8 +50,13 @@ __global__ __launch_bounds__(256) void latent_encode_kernel(
     acc += v * v;
   }
   const float kv_scale = rsqrtf(block_sum(acc, scratch) / static_cast<float>(kv_rank) + eps);
-  for (int i = threadIdx.x; i < kv_rank; i += blockDim.x)
-    record[i] = from_float<T>(to_float(latent[i]) * kv_scale * kv_weight[i]);
+  // (the second copy of the latent, keys contiguous: [page][dimension][place in the page])
+  T* turned = latents_t != nullptr ? latents_t + (slot / page_size) * kv_rank * page_size + slot % page_size : nullptr;
+  for (int i = threadIdx.x; i < kv_rank; i += blockDim.x) {
+    const T value = from_float<T>(to_float(latent[i]) * kv_scale * kv_weight[i]);
+    record[i] = value;
+    if (turned != nullptr) turned[static_cast<long>(i) * page_size] = value;
+  }
   const T* key = latent + kv_rank;
   const int half = rot_dims / 2;
   const int pos = positions[n];
@@ -73,10 +78,10 @@ __global__ __launch_bounds__(256) void latent_encode_kernel(
 }
 
 // ---- the rotated part of every query head, into its place behind the absorbed part --------------------------------------
-template <typename T>
+template <typename T, typename TY>
 __global__ void rotate_queries_kernel(const T* __restrict__ q, long tokens, int heads, int dim, int rot, int rot_dims,
                                       const float* __restrict__ table, int table_positions,
-                                      const int* __restrict__ positions, float* __restrict__ q_abs, int width, int at) {
+                                      const int* __restrict__ positions, TY* __restrict__ q_abs, int width, int at) {
   const long index = static_cast<long>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (index >= tokens * heads * rot) return;
   const int i = static_cast<int>(index % rot);
@@ -98,7 +103,7 @@ __global__ void rotate_queries_kernel(const T* __restrict__ q, long tokens, int 
       value = i < half ? u * c - v * s : v * c + u * s;
     }
   }
-  q_abs[row * width + at + i] = value;
+  q_abs[row * width + at + i] = from_float<TY>(value);
 }
 
 // ---- y[t, h, j] = sum_i x[t, h, i] w[h, i, j] ------------------------------------------------------------------------------
@@ -446,25 +451,34 @@ extern "C" {
 int akv_latent_encode(const void* down, int dtype, int tokens, int q_rank, int kv_rank, int rot, int rot_dims,
                       const float* q_weight, const float* kv_weight, float eps, const float* table, int table_positions,
                       const int* positions, const int* slot_map, void* cq, void* records, long record_slots,
-                      hipStream_t stream) {
+                      void* latents_t, int page_size, hipStream_t stream) {
   if (tokens <= 0) return 0;
-  if (rot_dims % 2 || rot_dims > rot || q_rank <= 0) return -2;
+  if (rot_dims % 2 || rot_dims > rot || q_rank <= 0 || (latents_t != nullptr && page_size <= 0)) return -2;
   AKV_DISPATCH(dtype, T, latent_encode_kernel<T><<<tokens, 256, 0, stream>>>(
                              static_cast<const T*>(down), q_rank, kv_rank, rot, rot_dims, q_weight, kv_weight, eps, table,
                              table_positions, positions, slot_map, static_cast<T*>(cq), static_cast<T*>(records),
-                             record_slots));
+                             record_slots, static_cast<T*>(latents_t), page_size));
   return AKV_LAUNCH_STATUS();
 }
 
 int akv_rotate_queries(const void* q, int dtype, long tokens, int heads, int dim, int rot, int rot_dims,
-                       const float* table, int table_positions, const int* positions, float* q_abs, int width, int at,
-                       hipStream_t stream) {
+                       const float* table, int table_positions, const int* positions, void* q_abs, int out_dtype,
+                       int width, int at, hipStream_t stream) {
   const long count = tokens * heads * rot;
   if (count <= 0) return 0;
   if (rot_dims % 2 || rot_dims > rot || at + rot > width) return -2;
-  AKV_DISPATCH(dtype, T, rotate_queries_kernel<T><<<static_cast<unsigned>((count + 255) / 256), 256, 0, stream>>>(
-                             static_cast<const T*>(q), tokens, heads, dim, rot, rot_dims, table, table_positions, positions,
-                             q_abs, width, at));
+  const unsigned blocks = static_cast<unsigned>((count + 255) / 256);
+  if (out_dtype == kF32) {
+    AKV_DISPATCH(dtype, T, rotate_queries_kernel<T, float><<<blocks, 256, 0, stream>>>(
+                               static_cast<const T*>(q), tokens, heads, dim, rot, rot_dims, table, table_positions, positions,
+                               static_cast<float*>(q_abs), width, at));
+  } else if (out_dtype == kBF16 && dtype == kBF16) {
+    rotate_queries_kernel<bf16_t, bf16_t><<<blocks, 256, 0, stream>>>(
+        static_cast<const bf16_t*>(q), tokens, heads, dim, rot, rot_dims, table, table_positions, positions,
+        static_cast<bf16_t*>(q_abs), width, at);
+  } else {
+    return -1;
+  }
   return AKV_LAUNCH_STATUS();
 }
 
@@ -485,6 +499,7 @@ int akv_heads_linear(const void* x, int x_dtype, long x_token_stride, long x_hea
   else if (x_dtype == kBF16 && w_dtype == kBF16 && y_dtype == kF32) AKV_HEADS(bf16_t, bf16_t, float);
   else if (x_dtype == kF32 && w_dtype == kBF16 && y_dtype == kBF16) AKV_HEADS(float, bf16_t, bf16_t);
   else if (x_dtype == kF32 && w_dtype == kBF16 && y_dtype == kF32) AKV_HEADS(float, bf16_t, float);
+  else if (x_dtype == kBF16 && w_dtype == kBF16 && y_dtype == kBF16) AKV_HEADS(bf16_t, bf16_t, bf16_t);
   else return -1;
 #undef AKV_HEADS
   return AKV_LAUNCH_STATUS();

@@ -37,7 +37,7 @@ class PartsKernels:
             except OSError as error:
                 raise KernelError(f"the kernel library {path} could not be loaded: {error}") from error
             for name in ("akv_embed_pairs", "akv_note_fed_tokens", "akv_norm_add_norm", "akv_latent_encode",
-                         "akv_rotate_queries", "akv_heads_linear", "akv_latent_attend", "akv_conv_silu",
+                         "akv_rotate_queries", "akv_heads_linear", "akv_latent_attend", "akv_latent_attend_mfma", "akv_conv_silu",
                          "akv_conv_state_update", "akv_selective_scan", "akv_route", "akv_gate_relu_squared",
                          "akv_parts_slot_layout"):
                 getattr(lib, name).restype = ctypes.c_int
@@ -117,10 +117,19 @@ class PartsKernels:
                                                     tokens, hidden, self._stream()), "norm_add_norm")
 
     # ---- attention over a compressed latent --------------------------------------------------------------------------
+    MATRIX_CORE_LATENTS = (128, 256, 512)
+
+    def latent_on_matrix_cores(self, heads: int, kv_rank: int, width: int, page_size: int, dtype) -> bool:
+        """Whether `latent_attend` has a matrix-core kernel for these sizes.  It reads a second copy of the latents with
+        the keys contiguous, which the layer then keeps beside the records (`latent_encode(..., latents_t=)`)."""
+        return (dtype == torch.bfloat16 and heads % 16 == 0 and width % 32 == 0 and kv_rank in self.MATRIX_CORE_LATENTS
+                and page_size % 8 == 0)
+
     def latent_encode(self, down, q_rank, kv_rank, rot, rot_dims, q_weight, kv_weight, eps, table, positions, slot_map,
-                      cq, records) -> None:
+                      cq, records, latents_t=None) -> None:
         """down [tokens, q_rank (+ kv_rank + rot)] -> cq = norm(q latent); with `records` [pages, 1, page, kv_rank + rot]
-        also the token's record: norm(kv latent), then the key part with its first `rot_dims` dimensions rotated."""
+        also the token's record: norm(kv latent), then the key part with its first `rot_dims` dimensions rotated; with
+        `latents_t` [pages, 1, kv_rank, page] the normed latent once more, keys contiguous."""
         tokens = down.shape[0]
         writes = records is not None
         self._dense(down, "down", None, (tokens, q_rank + (kv_rank + rot if writes else 0)))
@@ -138,18 +147,24 @@ class PartsKernels:
             self._dense(table, "table", torch.float32)
             if table.dim() != 3 or table.shape[1] != rot_dims // 2 or table.shape[2] != 2:
                 self._refuse(f"the rotation table must be [positions, {rot_dims // 2}, 2], got {tuple(table.shape)}")
+            if latents_t is not None:
+                self._dense(latents_t, "latents_t", down.dtype, (records.shape[0], 1, kv_rank, records.shape[2]))
         self._check(self._parts().akv_latent_encode(
             _ptr(down), self._code_of(down), tokens, q_rank, kv_rank, rot, rot_dims, _ptr(q_weight), _ptr(kv_weight),
             ctypes.c_float(eps), _ptr(table) if writes else ctypes.c_void_p(0), table.shape[0] if writes else 0,
             _ptr(positions), _ptr(slot_map) if writes else ctypes.c_void_p(0), _ptr(cq),
-            _ptr(records) if writes else ctypes.c_void_p(0), _long(slots), self._stream()), "latent_encode")
+            _ptr(records) if writes else ctypes.c_void_p(0), _long(slots),
+            _ptr(latents_t) if writes and latents_t is not None else ctypes.c_void_p(0),
+            records.shape[2] if writes else 0, self._stream()), "latent_encode")
 
     def rotate_queries(self, q, heads, dim, rot, rot_dims, table, positions, q_abs, at) -> None:
-        """q [tokens, heads * (dim + rot)] -> q_abs[:, :, at:at + rot] (float32): every head's last `rot` dimensions,
-        the first `rot_dims` of them rotated by the token's position."""
+        """q [tokens, heads * (dim + rot)] -> q_abs[:, :, at:at + rot] (float32, or bfloat16 like q): every head's last
+        `rot` dimensions, the first `rot_dims` of them rotated by the token's position."""
         tokens = q.shape[0]
         self._dense(q, "q", None, (tokens, heads * (dim + rot)))
-        self._dense(q_abs, "q_abs", torch.float32)
+        self._dense(q_abs, "q_abs")
+        if q_abs.dtype != torch.float32 and q_abs.dtype != q.dtype:
+            self._refuse(f"q_abs must be float32 or {q.dtype}, got {q_abs.dtype}")
         if q_abs.dim() != 3 or q_abs.shape[0] != tokens or q_abs.shape[1] != heads or at + rot > q_abs.shape[2]:
             self._refuse(f"q_abs must be [tokens, heads, at least {at + rot}], got {tuple(q_abs.shape)}")
         self._dense(table, "table", torch.float32)
@@ -158,7 +173,8 @@ class PartsKernels:
         self._dense(positions, "positions", torch.int32, (tokens,))
         self._check(self._parts().akv_rotate_queries(_ptr(q), self._code_of(q), _long(tokens), heads, dim, rot, rot_dims,
                                                      _ptr(table), table.shape[0], _ptr(positions), _ptr(q_abs),
-                                                     q_abs.shape[2], at, self._stream()), "rotate_queries")
+                                                     self._code_of(q_abs), q_abs.shape[2], at, self._stream()),
+                    "rotate_queries")
 
     def heads_linear(self, x, x_width: int, weight, y, y_width: int) -> None:
         """y[t, h, :outs] = x[t, h, :ins] W[h] for W [heads, ins, outs]: `x` is [tokens, heads, x_width] and `y`
@@ -170,18 +186,37 @@ class PartsKernels:
         self._dense(y, "y", None, (tokens, heads, y_width))
         if ins > x_width or outs > y_width:
             self._refuse(f"a product of {ins} -> {outs} per head does not fit rows of {x_width} and {y_width}")
+        above = getattr(self, "library_products_above", None)
+        if (above is not None and tokens > above and x.dtype == weight.dtype == y.dtype == torch.bfloat16):
+            # as with the plain products: many rows of bfloat16 go to the BLAS library, one batched product over the heads
+            torch.bmm(x[:, :, :ins].transpose(0, 1), weight, out=self._heads_scratch(heads, tokens, outs))
+            y[:, :, :outs].copy_(self._heads_scratch(heads, tokens, outs).transpose(0, 1))
+            return
         self._check(self._parts().akv_heads_linear(
             _ptr(x), self._code_of(x), _long(heads * x_width), _long(x_width), _ptr(weight), self._code_of(weight), _ptr(y),
             self._code_of(y), _long(heads * y_width), _long(y_width), tokens, heads, ins, outs, self._stream()),
             "heads_linear")
 
-    def latent_attend(self, q_abs, records, ctx, meta, heads, kv_rank, scale, window, out) -> None:
+    def _heads_scratch(self, heads: int, tokens: int, outs: int) -> torch.Tensor:
+        """Where a batched product over the heads leaves [heads, tokens, outs] before it is laid out by token."""
+        need = heads * tokens * outs
+        held = self.__dict__.get("_heads_buffer")
+        if held is None or held.numel() < need:
+            if torch.cuda.is_current_stream_capturing():
+                self._refuse("a recorded step needs more room for a product over the heads than the steps before it")
+            self.__dict__.setdefault("_heads_outgrown", []).append(held)
+            held = self.__dict__["_heads_buffer"] = torch.empty(max(need, 1 << 22), dtype=torch.bfloat16, device=self.device)
+        return held[:need].view(heads, tokens, outs)
+
+    def latent_attend(self, q_abs, records, ctx, meta, heads, kv_rank, scale, window, out, latents_t=None) -> None:
         """Every head of every token attends the records [kv_rank + rot] of its request's last `window` tokens (all,
         if None): softmax((q_abs . record) * scale), then the weighted sum of the records' first kv_rank dimensions
-        -> out [tokens, heads, kv_rank] float32."""
+        -> out [tokens, heads, kv_rank].  q_abs and out are float32 - or, with `latents_t` (the layer's second copy of
+        the latents, see `latent_on_matrix_cores`), bfloat16: the matrix-core kernel."""
         tokens, width = q_abs.shape[0], q_abs.shape[2]
-        self._dense(q_abs, "q_abs", torch.float32, (tokens, heads, width))
-        self._dense(out, "out", torch.float32, (tokens, heads, kv_rank))
+        mfma = latents_t is not None
+        self._dense(q_abs, "q_abs", torch.bfloat16 if mfma else torch.float32, (tokens, heads, width))
+        self._dense(out, "out", q_abs.dtype, (tokens, heads, kv_rank))
         self._dense(records, "records")
         if records.dim() != 4 or records.shape[1] != 1 or records.shape[3] != width:
             self._refuse(f"records must be [pages, 1, page, {width}], got {tuple(records.shape)}")
@@ -197,6 +232,16 @@ class PartsKernels:
             self._refuse("the block table has fewer rows than the step has requests")
         if ctx.max_seq_len > meta.width * records.shape[2]:
             self._refuse("a request is longer than its row of the block table")
+        if mfma:
+            if not self.latent_on_matrix_cores(heads, kv_rank, width, records.shape[2], records.dtype):
+                self._refuse("the matrix-core attention over latents does not take these sizes")
+            self._dense(latents_t, "latents_t", torch.bfloat16, (records.shape[0], 1, kv_rank, records.shape[2]))
+            self._check(self._parts().akv_latent_attend_mfma(
+                _ptr(q_abs), _ptr(records), _ptr(latents_t), _ptr(ctx.seq_of_token), _ptr(ctx.positions),
+                _ptr(meta.block_table), _ptr(meta.rows), meta.width, _ptr(out), tokens, heads, kv_rank, width,
+                records.shape[2], _long(records.shape[0]), ctypes.c_float(scale), int(window) if window is not None else 0,
+                self._stream()), "latent_attend on the matrix cores")
+            return
         self._check(self._parts().akv_latent_attend(
             _ptr(q_abs), _ptr(records), self._code_of(records), _ptr(ctx.seq_of_token), _ptr(ctx.positions),
             _ptr(meta.block_table), _ptr(meta.rows), meta.width, _ptr(out), tokens, heads, kv_rank, width, records.shape[2],

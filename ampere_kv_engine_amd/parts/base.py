@@ -274,6 +274,11 @@ class KernelSet:
         """`linear_after_norm(stream, delta, norm_weight, eps, stream_out, weight, out, bias=)` exists for this product."""
         return False
 
+    def latent_on_matrix_cores(self, heads: int, kv_rank: int, width: int, page_size: int, dtype) -> bool:
+        """`latent_attend(..., latents_t=)` exists for these sizes: a kernel that wants the latents a second time with the
+        keys contiguous (`latent_encode(..., latents_t=)` writes them), and bfloat16 queries."""
+        return False
+
     def measure_products(self, *args, **kwargs) -> dict:
         """Times the candidates for every prepared product once (`EngineConfig.product_choices = "measure"`)."""
         return {}

@@ -53,6 +53,14 @@ class LatentAttention(Part):
         self.out = Linear(runtime, self.heads * self.vdim, [self.hidden], ["o"])
         self.position = build_part("position", part("rope_half", head_dim=self.rot_dims, theta=float(spec["rotary_base"])),
                                    runtime)
+        # where the kernel set has a matrix-core kernel for these sizes the layer keeps the latents twice: inside the
+        # records, and once more with the keys contiguous, as that kernel's second product reads them
+        # (the copy is kept by the layer that writes the records, for whichever of their readers has such a kernel:
+        # `reader_heads`, the head counts of all layers that read this layer's cache)
+        fits = lambda heads: bool(runtime.kernels.latent_on_matrix_cores(int(heads), self.kv_rank, self.record,
+                                                                         runtime.page_size, runtime.dtype))
+        self.on_matrix_cores = fits(self.heads)
+        self.keeps_turned = any(fits(heads) for heads in spec.get("reader_heads", (self.heads,)))
         self.q_norm_weight = self.kv_norm_weight = None
         self.key_up = self.value_up = None      # [heads, dim, kv_rank] and [heads, kv_rank, vdim], as the per-head products read them
         self._bytes = 0
@@ -93,8 +101,9 @@ class LatentAttention(Part):
 
     # ---- cache ------------------------------------------------------------------------------------------------------
     def cache_request(self):
-        """One record per token and no values: what a head multiplies its weights with is the record's first part."""
-        return PagedKV(1, self.record, self.cache_window, value_dim=0)
+        """One record per token and no values: what a head multiplies its weights with is the record's first part -
+        kept a second time in the values' layout where the matrix cores read it."""
+        return PagedKV(1, self.record, self.cache_window, value_dim=self.kv_rank if self.keeps_turned else 0)
 
     # ---- one step ---------------------------------------------------------------------------------------------------
     def forward(self, x, ctx, cache, writes_cache: bool = True):
@@ -108,16 +117,19 @@ class LatentAttention(Part):
         down = ctx.arena.take((tokens, self.down.total_out), dtype)
         self.down.forward(x, down)
         cq = ctx.arena.take((tokens, self.q_rank), dtype)
+        turned = cache.v if self.on_matrix_cores else None
         k.latent_encode(down, self.q_rank, self.kv_rank, self.rot, self.rot_dims, self.q_norm_weight, self.kv_norm_weight,
-                        self.eps, self.position.table, ctx.positions, meta.slot_map, cq, cache.k if writes_cache else None)
+                        self.eps, self.position.table, ctx.positions, meta.slot_map, cq, cache.k if writes_cache else None,
+                        latents_t=cache.v if writes_cache else None)
         q = ctx.arena.take((tokens, self.heads * (self.dim + self.rot)), dtype)
         self.up_q.forward(cq, q)
-        q_abs = ctx.arena.take((tokens, self.heads, self.record), torch.float32)
+        between = dtype if turned is not None else torch.float32      # the matrix cores take their queries in bfloat16
+        q_abs = ctx.arena.take((tokens, self.heads, self.record), between)
         k.heads_linear(q.view(tokens, self.heads, self.dim + self.rot), self.dim + self.rot, self.key_up, q_abs, self.record)
         k.rotate_queries(q, self.heads, self.dim, self.rot, self.rot_dims, self.position.table, ctx.positions, q_abs,
                          self.kv_rank)
-        mixed = ctx.arena.take((tokens, self.heads, self.kv_rank), torch.float32)
-        k.latent_attend(q_abs, cache.k, ctx, meta, self.heads, self.kv_rank, self.scale, self.window, mixed)
+        mixed = ctx.arena.take((tokens, self.heads, self.kv_rank), between)
+        k.latent_attend(q_abs, cache.k, ctx, meta, self.heads, self.kv_rank, self.scale, self.window, mixed, latents_t=turned)
         values = ctx.arena.take((tokens, self.heads, self.vdim), dtype)
         k.heads_linear(mixed, self.kv_rank, self.value_up, values, self.vdim)
         out = ctx.arena.take((tokens, self.hidden), dtype)

@@ -41,7 +41,17 @@ KERANEX_B = dict(
         dict(type="latent_attention", mixer=LATENT(2, 16, 4, 8, 24, 8, 1, 0.25, 50.0), mlp=None),
         dict(type="latent_attention", mixer=LATENT(4, 16, 16, 16, 72, 32, 19, 0.25, 10000.0, kv_from=0), mlp=MOE(3, 1, 3, 1, 40)),
     ])
-KERANEX = {"A": (KERANEX_A, 11, 4), "B": (KERANEX_B, 12, 8)}        # config, weight seed, page size
+# Heads in multiples of 16 and latents of 128: the sizes at which, in bfloat16, the attention runs on the matrix cores
+# and the layer keeps its latents a second time - for the reader of 32 heads too, whose window is the narrower one.
+KERANEX_C = dict(
+    architecture="Keranex", vocab=300, width=128, norm=dict(eps=1e-5),
+    embedding=dict(bigram=dict(buckets=64, mul_prev=7, mul_cur=9)),
+    layers=[
+        dict(type="latent_attention", mixer=LATENT(16, 32, 32, 32, 128, 64, 40, 0.12, 10000.0), mlp=MOE(4, 2, 2, 1, 32)),
+        dict(type="mamba1", mixer=SCAN(128, 8, 8, 4), mlp=None),
+        dict(type="latent_attention", mixer=LATENT(32, 16, 32, 16, 128, 48, 24, 0.15, 10000.0, kv_from=0), mlp=MOE(4, 2, 2, 1, 32)),
+    ])
+KERANEX = {"A": (KERANEX_A, 11, 4), "B": (KERANEX_B, 12, 8), "C": (KERANEX_C, 13, 16)}        # config, weight seed, page size
 
 LENGTHS = {"a": 70, "b": 45, "e": 33, "d": 96, "c": 61, "f": 27}
 PROMPTS = {"a": 40, "b": 45, "c": 30, "d": 20, "e": 1, "f": 20}

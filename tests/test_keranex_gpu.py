@@ -266,6 +266,28 @@ def test_latent_attention_over_records(hip, dtype, heads, kv_rank, rot, page, po
         torch.testing.assert_close(out[first:first + count].cpu(), want, rtol=1e-4, atol=1e-4)
 
 
+@pytest.mark.parametrize("heads,kv_rank,rot,page", [(16, 128, 32, 16), (32, 512, 64, 16), (16, 256, 32, 8), (48, 128, 64, 32)])
+@pytest.mark.parametrize("portions,window", [([(0, 1)], 5), ([(0, 70)], 19), ([(64, 1), (17, 1), (0, 1)], 16), ([(31, 2)], 32),
+                                             ([(5, 7), (63, 2), (130, 1), (0, 70)], 40), ([(200, 3), (0, 9)], None),
+                                             ([(500, 40)], 300)])
+def test_latent_attention_on_the_matrix_cores(hip, heads, kv_rank, rot, page, portions, window):
+    """bfloat16 queries and records; the latents a second time with the keys contiguous.  Against the plain function on
+    the same rounded operands."""
+    assert hip.latent_on_matrix_cores(heads, kv_rank, kv_rank + rot, page, torch.bfloat16)
+    pages, table, records = records_case(torch.bfloat16, kv_rank, rot, page, portions, window, 51)
+    turned = pages[:, :, :, :kv_rank].transpose(2, 3).contiguous()
+    ctx = step_of(portions)
+    meta = SimpleNamespace(block_table=table.cuda(), width=table.shape[1], window=window, rows=None)
+    q_abs = rand(ctx.num_tokens, heads, kv_rank + rot, seed=52, scale=0.4, dtype=torch.bfloat16)
+    out = torch.empty(ctx.num_tokens, heads, kv_rank, dtype=torch.bfloat16, device="cuda")
+    hip.latent_attend(q_abs.cuda(), pages.cuda(), ctx, meta, heads, kv_rank, 0.2, window, out, latents_t=turned.cuda())
+    for r, (history, count) in enumerate(portions):
+        first = ctx.host_q_start[r]
+        want = plain.attend_records(q_abs[first:first + count].float(), records[r].float(),
+                                    list(range(history, history + count)), window, 0.2, kv_rank)
+        torch.testing.assert_close(out[first:first + count].cpu().float(), want, rtol=1e-2, atol=1e-2)
+
+
 @pytest.mark.parametrize("window,page", [(16, 16), (17, 16), (40, 16), (5, 4), (64, 8), (1, 4)])
 @pytest.mark.parametrize("history", [0, 3, 63, 64, 200])
 def test_one_key_stands_out_just_inside_and_just_outside_the_window(hip, window, page, history):

@@ -286,7 +286,7 @@ class TorchKernels(KernelSet):
         return torch.cat((u * cos - v * sin, v * cos + u * sin, x[..., rot_dims:]), dim=-1)
 
     def latent_encode(self, down, q_rank, kv_rank, rot, rot_dims, q_weight, kv_weight, eps, table, positions, slot_map,
-                      cq, records):
+                      cq, records, latents_t=None):
         d = down.float()
         ql = d[:, :q_rank]
         cq.copy_((ql * torch.rsqrt((ql * ql).mean(-1, keepdim=True) + eps) * q_weight).to(cq.dtype))
@@ -306,7 +306,7 @@ class TorchKernels(KernelSet):
         heads, ins, outs = weight.shape
         y[..., :outs] = torch.einsum("thi,hio->tho", x[..., :ins].float(), weight.float()).to(y.dtype)
 
-    def latent_attend(self, q_abs, records, ctx, meta, heads, kv_rank, scale, window, out):
+    def latent_attend(self, q_abs, records, ctx, meta, heads, kv_rank, scale, window, out, latents_t=None):
         page_size = records.shape[2]
         table = meta.block_table.cpu()
         if getattr(meta, "rows", None) is not None:
