@@ -47,11 +47,13 @@ int akv_latent_attend(const float* q_abs, const void* records, int dtype, const 
 // The same on the matrix cores, for bfloat16, heads that are a multiple of 16, records a multiple of 32 wide, latents
 // of 128, 256 or 512 and pages of a multiple of 8 tokens (-2 otherwise).  `latents_t` [pages, kv_rank, page]: the
 // records' first kv_rank dimensions once more, keys contiguous.  q_abs [tokens, heads, width] and out [tokens, heads,
-// kv_rank] are bfloat16.
+// kv_rank] are bfloat16.  With `segments` > 1 a token's keys are cut into runs of `segment` keys (a multiple of 32, at
+// absolute positions, counted from the run that holds its window's first key; the caller gives as many as the longest
+// span needs), a wave each, whose shares meet in `parts` [tokens * heads * segments * (kv_rank + 2)] and are merged.
 int akv_latent_attend_mfma(const void* q_abs, const void* records, const void* latents_t, const int* seq_of_token,
                            const int* positions, const int* block_table, const int* table_rows, int table_width,
                            void* out, int tokens, int heads, int kv_rank, int width, int page_size, long num_pages,
-                           float scale, int window, hipStream_t stream);
+                           float scale, int window, int segment, int segments, float* parts, hipStream_t stream);
 
 // ---- selective scan (selective_scan.hip) ----------------------------------------------------------------------------
 // x [tokens, channels] at `x_stride` per token; state [slots, state_stride] float32 holds (taps - 1) x channels at
@@ -68,9 +70,9 @@ int akv_selective_scan(const void* x, int dtype, const float* dt, const float* b
                        const int* seq_slots, void* out, int seqs, int channels, int n_state, hipStream_t stream);
 
 // ---- routed feed-forward (routed.hip) -------------------------------------------------------------------------------
-// gates [tokens, experts] float32: the softmax score of the chosen experts, 0 elsewhere
-int akv_route(const void* x, int dtype, const float* router, float* gates, int tokens, int hidden, int experts,
-              int top, int groups, int keep, hipStream_t stream);
+// logits [tokens, experts] float32 -> gates [tokens, experts] float32: the softmax score of the chosen experts, 0 elsewhere
+int akv_route(const float* logits, float* gates, int tokens, int experts, int top, int groups, int keep,
+              hipStream_t stream);
 // act[t, e * ff + j] = gates[t, e] * relu(up[t, e * ff + j])^2
 int akv_gate_relu_squared(const void* up, const float* gates, void* act, int dtype, long tokens, int experts, int ff,
                           hipStream_t stream);

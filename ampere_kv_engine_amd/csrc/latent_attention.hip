@@ -271,12 +271,13 @@ __global__ __launch_bounds__(256) void latent_attend_mfma_kernel(
     const bf16_t* __restrict__ q_abs, const bf16_t* __restrict__ records, const bf16_t* __restrict__ latents_t,
     const int* __restrict__ seq_of_token, const int* __restrict__ positions, const int* __restrict__ block_table,
     const int* __restrict__ table_rows, int table_width, bf16_t* __restrict__ out, long tiles, int heads, int width,
-    int page_size, long num_pages, float scale_log2, int window) {
+    int page_size, long num_pages, float scale_log2, int window, int segment, int segments, float* __restrict__ parts) {
   extern __shared__ unsigned char lds_bytes[];
   constexpr int kv_rank = VT * 16;
   const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
   const long tile = static_cast<long>(blockIdx.x) * (blockDim.x / kWave) + wave;
   if (tile >= tiles) return;
+  const int part = blockIdx.y;            // which run of `segment` keys (aligned to absolute positions) this wave takes
   const int rho = lane & 15, g = lane >> 4;
   const long n = tile * 16 / heads;                         // the tile's token (heads are a multiple of 16)
   const int r = table_rows != nullptr ? table_rows[seq_of_token[n]] : seq_of_token[n];
@@ -307,10 +308,41 @@ __global__ __launch_bounds__(256) void latent_attend_mfma_kernel(
   bool poisoned = lost;
   const int steps32 = width / 32;
 
-  for (int base = lowest & ~31; base <= pos; base += 32) {
+  // keys this wave looks at: all the token may see, or - where the launch cuts them - its run of them.  Runs are
+  // counted from the window's first key rounded down to a run's size, so a token's cut depends on its position alone.
+  int first_base = lowest & ~31, last_key = pos;
+  if (segments > 1) {
+    const int run0 = lowest / segment * segment + part * segment;
+    first_base = max(first_base, run0);
+    last_key = min(pos, run0 + segment - 1);
+  }
+  constexpr int kAhead = 6;               // operands asked for before the first of them is multiplied
+
+  for (int base = first_base; base <= last_key; base += 32) {
     const bool edge = base < lowest || base + 31 > pos;
-    // ---- scores: two tiles of 16 keys ---------------------------------------------------------------------------
-    floatx4 s[2];
+    // ---- this step's latents (needed after the softmax): asked for first ------------------------------------------------
+    const int first_key = base + g * 8;
+    long value_page = safe_page;
+    int value_at = 0;
+    uint32_t keep[4] = {0u, 0u, 0u, 0u};          // which of the 8 keys count (others may hold anything)
+    if (first_key + 7 >= lowest && first_key <= pos) {
+      const long page = table[first_key / page_size];
+      if (page >= 0 && page < num_pages) {
+        value_page = page;
+        value_at = first_key % page_size;
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (first_key + e >= lowest && first_key + e <= pos) keep[e >> 1] |= (e & 1) ? 0xffff0000u : 0x0000ffffu;
+      } else {
+        poisoned = true;
+      }
+    }
+    const bf16_t* values = latents_t + (value_page * kv_rank + rho) * page_size + value_at;
+    uintx4 vreg[VT];
+#pragma unroll
+    for (int dt = 0; dt < VT; ++dt) vreg[dt] = *reinterpret_cast<const uintx4*>(values + static_cast<long>(dt) * 16 * page_size);
+    // ---- scores: two tiles of 16 keys, their operands fetched kAhead at a time ------------------------------------------
+    const uintx4* rows[2];
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       const int key = base + (rho >> 2) * 8 + j * 4 + (rho & 3);
@@ -320,11 +352,24 @@ __global__ __launch_bounds__(256) void latent_attend_mfma_kernel(
         if (page < 0 || page >= num_pages) poisoned = true;
         else slot = page * page_size + key % page_size;
       }
-      const uintx4* row = reinterpret_cast<const uintx4*>(records + slot * width) + g;
-      floatx4 acc = floatx4{0.f, 0.f, 0.f, 0.f};
-      for (int t = 0; t < steps32; ++t)
-        acc = mfma16(row[t * 4], *reinterpret_cast<const uintx4*>(q_mine + t * 64), acc);
-      s[j] = acc;
+      rows[j] = reinterpret_cast<const uintx4*>(records + slot * width) + g;
+    }
+    floatx4 s[2] = {floatx4{0.f, 0.f, 0.f, 0.f}, floatx4{0.f, 0.f, 0.f, 0.f}};
+    for (int t0 = 0; t0 < steps32; t0 += kAhead) {
+      uintx4 k0[kAhead], k1[kAhead], qq[kAhead];
+#pragma unroll
+      for (int u = 0; u < kAhead; ++u) {
+        const int t = min(t0 + u, steps32 - 1);     // (beyond the record: its last operand again, against zeros)
+        k0[u] = rows[0][t * 4];
+        k1[u] = rows[1][t * 4];
+        qq[u] = *reinterpret_cast<const uintx4*>(q_mine + t * 64);
+        if (t0 + u >= steps32) qq[u] = uintx4{0u, 0u, 0u, 0u};
+      }
+#pragma unroll
+      for (int u = 0; u < kAhead; ++u) {
+        s[0] = mfma16(k0[u], qq[u], s[0]);
+        s[1] = mfma16(k1[u], qq[u], s[1]);
+      }
     }
     if (edge) {
 #pragma unroll
@@ -365,29 +410,31 @@ __global__ __launch_bounds__(256) void latent_attend_mfma_kernel(
       for (int dt = 0; dt < VT; ++dt) o[dt] *= correction;
     }
     // ---- O^T += C^T P^T: this lane's 8 keys base + g * 8 .. + 7 of dimension dt * 16 + rho ---------------------------
-    const int first_key = base + g * 8;
-    long value_page = safe_page;
-    int value_at = 0;
-    uint32_t keep[4] = {0u, 0u, 0u, 0u};          // which of the 8 keys count (others may hold anything)
-    if (first_key + 7 >= lowest && first_key <= pos) {
-      const long page = table[first_key / page_size];
-      if (page >= 0 && page < num_pages) {
-        value_page = page;
-        value_at = first_key % page_size;
-#pragma unroll
-        for (int e = 0; e < 8; ++e)
-          if (first_key + e >= lowest && first_key + e <= pos) keep[e >> 1] |= (e & 1) ? 0xffff0000u : 0x0000ffffu;
-      } else {
-        poisoned = true;
-      }
-    }
-    const bf16_t* values = latents_t + (value_page * kv_rank + rho) * page_size + value_at;
 #pragma unroll
     for (int dt = 0; dt < VT; ++dt) {
-      uintx4 v = *reinterpret_cast<const uintx4*>(values + static_cast<long>(dt) * 16 * page_size);
+      uintx4 v = vreg[dt];
       if (edge) v = uintx4{v[0] & keep[0], v[1] & keep[1], v[2] & keep[2], v[3] & keep[3]};
       o[dt] = mfma16(v, p_low, mfma16(v, p_high, o[dt]));
     }
+  }
+  if (segments > 1) {
+    // this run's share: the sums as they are, with the maximum and the sum of weights they were formed against, for the
+    // merge.  parts: [tile][part][16 columns][kv_rank + 2]
+    float* mine = parts + ((tile * segments + part) * 16 + rho) * (kv_rank + 2);
+    l += __shfl_xor(l, 16, kWave);
+    l += __shfl_xor(l, 32, kWave);
+    const bool bad = __any(poisoned);
+#pragma unroll
+    for (int dt = 0; dt < VT; ++dt) {
+      floatx4 v = o[dt];
+      if (bad) v = floatx4{__uint_as_float(kPoison), __uint_as_float(kPoison), __uint_as_float(kPoison), __uint_as_float(kPoison)};
+      store4<float>(mine + dt * 16 + g * 4, v);
+    }
+    if (g == 0) {
+      mine[kv_rank] = m;
+      mine[kv_rank + 1] = l;
+    }
+    return;
   }
   l += __shfl_xor(l, 16, kWave);
   l += __shfl_xor(l, 32, kWave);
@@ -402,11 +449,35 @@ __global__ __launch_bounds__(256) void latent_attend_mfma_kernel(
   }
 }
 
+// The runs' shares of a column added up: each was formed against its own maximum m; against the largest of them
+// every share counts exp2(m - M) times.  One wave per (tile, column); a lane owns dimensions lane, lane + 64, ...
+__global__ __launch_bounds__(64) void latent_merge_kernel(const float* __restrict__ parts, bf16_t* __restrict__ out,
+                                                          int segments, int kv_rank) {
+  const long column = blockIdx.x;                   // tile * 16 + rho
+  const long tile = column / 16, rho = column % 16;
+  const int lane = threadIdx.x;
+  float top = -INFINITY;
+  for (int p = 0; p < segments; ++p) top = fmaxf(top, parts[((tile * segments + p) * 16 + rho) * (kv_rank + 2) + kv_rank]);
+  float total = 0.f;
+  for (int p = 0; p < segments; ++p) {
+    const float* share = parts + ((tile * segments + p) * 16 + rho) * (kv_rank + 2);
+    if (share[kv_rank] != -INFINITY) total += share[kv_rank + 1] * __builtin_amdgcn_exp2f(share[kv_rank] - top);
+  }
+  for (int d = lane; d < kv_rank; d += kWave) {
+    float acc = 0.f;
+    for (int p = 0; p < segments; ++p) {
+      const float* share = parts + ((tile * segments + p) * 16 + rho) * (kv_rank + 2);
+      if (share[kv_rank] != -INFINITY) acc += share[d] * __builtin_amdgcn_exp2f(share[kv_rank] - top);
+    }
+    out[column * kv_rank + d] = from_float<bf16_t>(acc / total);
+  }
+}
+
 template <int VT>
 int launch_attend_mfma(const void* q_abs, const void* records, const void* latents_t, const int* seq_of_token,
                        const int* positions, const int* block_table, const int* table_rows, int table_width, void* out,
                        long tiles, int heads, int width, int page_size, long num_pages, float scale, int window,
-                       hipStream_t stream) {
+                       int segment, int segments, float* parts, hipStream_t stream) {
   constexpr int waves = 4;
   const size_t lds = static_cast<size_t>(waves) * 16 * (width / 8 + 1) * 16;
   auto kernel = latent_attend_mfma_kernel<VT>;
@@ -414,10 +485,14 @@ int launch_attend_mfma(const void* q_abs, const void* records, const void* laten
   if (lds > 64 * 1024 && hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                              static_cast<int>(lds)) != hipSuccess)
     return -2;
-  kernel<<<static_cast<unsigned>((tiles + waves - 1) / waves), waves * kWave, lds, stream>>>(
+  kernel<<<dim3(static_cast<unsigned>((tiles + waves - 1) / waves), segments), waves * kWave, lds, stream>>>(
       static_cast<const bf16_t*>(q_abs), static_cast<const bf16_t*>(records), static_cast<const bf16_t*>(latents_t),
       seq_of_token, positions, block_table, table_rows, table_width, static_cast<bf16_t*>(out), tiles, heads, width,
-      page_size, num_pages, scale * 1.4426950408889634f, window);
+      page_size, num_pages, scale * 1.4426950408889634f, window, segment, segments, parts);
+  const int status = AKV_LAUNCH_STATUS();
+  if (status != 0 || segments == 1) return status;
+  latent_merge_kernel<<<static_cast<unsigned>(tiles * 16), kWave, 0, stream>>>(parts, static_cast<bf16_t*>(out), segments,
+                                                                              VT * 16);
   return AKV_LAUNCH_STATUS();
 }
 
@@ -489,7 +564,8 @@ int akv_heads_linear(const void* x, int x_dtype, long x_token_stride, long x_hea
   if (ins <= 0 || outs <= 0) return -2;
   const size_t lds_bytes = static_cast<size_t>(ins) * kHeadTokens * 4;
   if (lds_bytes > 64 * 1024) return -2;
-  const int threads = outs >= 256 ? 256 : (outs + kWave - 1) / kWave * kWave;
+  // few tokens: a head's matrix is the work, cut over more blocks (a wave each); many: blocks of up to four waves
+  const int threads = tokens <= 2 * kHeadTokens ? kWave : outs >= 256 ? 256 : (outs + kWave - 1) / kWave * kWave;
   const dim3 grid((tokens + kHeadTokens - 1) / kHeadTokens, heads, (outs + threads - 1) / threads);
 #define AKV_HEADS(TX, TW, TY)                                                                                       \
   heads_linear_kernel<TX, TW, TY><<<grid, threads, lds_bytes, stream>>>(                                            \
@@ -533,13 +609,14 @@ int akv_latent_attend(const float* q_abs, const void* records, int dtype, const 
 int akv_latent_attend_mfma(const void* q_abs, const void* records, const void* latents_t, const int* seq_of_token,
                            const int* positions, const int* block_table, const int* table_rows, int table_width,
                            void* out, int tokens, int heads, int kv_rank, int width, int page_size, long num_pages,
-                           float scale, int window, hipStream_t stream) {
+                           float scale, int window, int segment, int segments, float* parts, hipStream_t stream) {
   if (tokens <= 0) return 0;
   if (heads % 16 || width % 32 || kv_rank % 16 || kv_rank > width || page_size % 8) return -2;
+  if (segments < 1 || (segments > 1 && (segment < 32 || segment % 32 || parts == nullptr))) return -2;
   const long tiles = static_cast<long>(tokens) * heads / 16;
 #define AKV_MFMA(VT)                                                                                                   \
   return launch_attend_mfma<VT>(q_abs, records, latents_t, seq_of_token, positions, block_table, table_rows, table_width, \
-                                out, tiles, heads, width, page_size, num_pages, scale, window, stream)
+                                out, tiles, heads, width, page_size, num_pages, scale, window, segment, segments, parts, stream)
   if (kv_rank == 128) AKV_MFMA(8);
   if (kv_rank == 256) AKV_MFMA(16);
   if (kv_rank == 512) AKV_MFMA(32);

@@ -1,5 +1,5 @@
-// A routed feed-forward's token-wise kernels: the router (float32 logits, softmax over all experts, the choice
-// restricted to the best groups of neighbouring experts) and the experts' activation times the router's weight.
+// A routed feed-forward's token-wise kernels: the choice of experts from the router's float32 logits (softmax over all
+// experts, the choice restricted to the best groups of neighbouring experts) and the experts' activation times the router's weight.
 
 #include "common.h"
 #include "api_parts.h"
@@ -8,13 +8,12 @@ using namespace akv;
 
 namespace {
 
-// One wave per token.  scores = softmax(router x); a group's score is its best expert's; only experts of the `keep`
-// best groups can be chosen; the `top` best of those are, each weighted by its own score (the weights are not
-// renormalised).  Equal scores go to the lower index.  gates[t, e] = score of a chosen expert, 0 of any other.
-template <typename T>
-__global__ __launch_bounds__(256) void route_kernel(const T* __restrict__ x, const float* __restrict__ router,
-                                                    float* __restrict__ gates, int tokens, int hidden, int experts,
-                                                    int top, int groups, int keep) {
+// One wave per token, from the router's logits (a product of the engine's, float32 sums).  scores = softmax(logits);
+// a group's score is its best expert's; only experts of the `keep` best groups can be chosen; the `top` best of those
+// are, each weighted by its own score (the weights are not renormalised).  Equal scores go to the lower index.
+// gates[t, e] = score of a chosen expert, 0 of any other.
+__global__ __launch_bounds__(256) void route_kernel(const float* __restrict__ logits, float* __restrict__ gates,
+                                                    int tokens, int experts, int top, int groups, int keep) {
   extern __shared__ float lds[];
   const int waves = blockDim.x / kWave, wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
   const int n = blockIdx.x * waves + wave;
@@ -22,20 +21,18 @@ __global__ __launch_bounds__(256) void route_kernel(const T* __restrict__ x, con
   float* score = lds + static_cast<size_t>(wave) * (2 * experts + groups);   // [experts]
   float* open = score + experts;        // [experts]: 1 while the expert may still be chosen, 2 once it is chosen, 0 shut
   float* best = open + experts;         // [groups]
-  const T* row = x + static_cast<size_t>(n) * hidden;
-  for (int e = 0; e < experts; ++e) {
-    const float* w = router + static_cast<size_t>(e) * hidden;
-    float acc = 0.f;
-    for (int i = lane; i < hidden; i += kWave) acc = fmaf(to_float(row[i]), w[i], acc);
-    acc = wave_sum(acc);
-    if (lane == 0) score[e] = acc;
+  float highest = -INFINITY;
+  for (int e = lane; e < experts; e += kWave) {
+    const float z = logits[static_cast<size_t>(n) * experts + e];
+    score[e] = z;
+    highest = fmaxf(highest, z);
   }
+  highest = wave_max(highest);
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   if (lane == 0) {       // a few dozen numbers: one lane does the choosing
-    float highest = -INFINITY, total = 0.f;
-    for (int e = 0; e < experts; ++e) highest = fmaxf(highest, score[e]);
+    float total = 0.f;
     for (int e = 0; e < experts; ++e) {
       score[e] = expf(score[e] - highest);
       total += score[e];
@@ -95,15 +92,15 @@ __global__ void gate_relu_squared_kernel(const T* __restrict__ up, const float* 
 
 extern "C" {
 
-int akv_route(const void* x, int dtype, const float* router, float* gates, int tokens, int hidden, int experts,
-              int top, int groups, int keep, hipStream_t stream) {
+int akv_route(const float* logits, float* gates, int tokens, int experts, int top, int groups, int keep,
+              hipStream_t stream) {
   if (tokens <= 0) return 0;
   if (experts <= 0 || groups <= 0 || experts % groups || keep <= 0 || keep > groups || top <= 0 || top > experts) return -2;
   const int waves = 4;
   const size_t lds_bytes = static_cast<size_t>(waves) * (2 * experts + groups) * 4;
   if (lds_bytes > 64 * 1024) return -2;
-  AKV_DISPATCH(dtype, T, route_kernel<T><<<(tokens + waves - 1) / waves, waves * kWave, lds_bytes, stream>>>(
-                             static_cast<const T*>(x), router, gates, tokens, hidden, experts, top, groups, keep));
+  route_kernel<<<(tokens + waves - 1) / waves, waves * kWave, lds_bytes, stream>>>(logits, gates, tokens, experts, top,
+                                                                                   groups, keep);
   return AKV_LAUNCH_STATUS();
 }
 

@@ -67,6 +67,11 @@ __global__ __launch_bounds__(256) void conv_state_update_kernel(const T* __restr
 }
 
 // ---- the scan: a thread owns a channel of a request, its row of S in registers, and walks the portion's tokens ------
+// Tokens are taken kScanAhead at a time: their inputs are asked for together (a token's own arithmetic is short, and
+// one trip to memory per token would be all a long portion's time), and the wave lays the tokens' B and C, which all
+// channels share, into LDS once.
+constexpr int kScanAhead = 8;
+
 template <typename T, int NS>
 __global__ __launch_bounds__(64) void selective_scan_kernel(const T* __restrict__ x, const float* __restrict__ dt,
                                                             const float* __restrict__ bc, const T* __restrict__ z,
@@ -75,36 +80,59 @@ __global__ __launch_bounds__(64) void selective_scan_kernel(const T* __restrict_
                                                             long state_stride, const int* __restrict__ q_start,
                                                             const int* __restrict__ seq_slots, T* __restrict__ out,
                                                             int channels, int n_state) {
+  extern __shared__ float shared_bc[];                // [kScanAhead][2 * n_state]
   const int r = blockIdx.x;
   const int c = blockIdx.y * blockDim.x + threadIdx.x;
-  if (c >= channels) return;
-  float* kept = state + static_cast<long>(seq_slots[r]) * state_stride + static_cast<long>(c) * n_state;
+  const bool works = c < channels;
+  const int cc = works ? c : channels - 1;            // (a lane beyond the channels keeps the wave's steps and stores nothing)
+  float* kept = state + static_cast<long>(seq_slots[r]) * state_stride + static_cast<long>(cc) * n_state;
   float S[NS], A[NS];
 #pragma unroll
   for (int n = 0; n < NS; ++n) {
     S[n] = n < n_state ? kept[n] : 0.f;
-    A[n] = n < n_state ? a[static_cast<long>(c) * n_state + n] : 0.f;
+    A[n] = n < n_state ? a[static_cast<long>(cc) * n_state + n] : 0.f;
   }
-  const float skip = d[c];
-  const int last = q_start[r + 1];
-  for (int t = q_start[r]; t < last; ++t) {
-    const float xv = to_float(x[static_cast<long>(t) * channels + c]);
-    const float step = softplus(dt[static_cast<long>(t) * channels + c]);
-    const float gate = to_float(z[t * z_stride + c]);
-    const float* B = bc + static_cast<long>(t) * 2 * n_state;
-    const float* C = B + n_state;
-    const float drive = step * xv;
-    float y = 0.f;
-#pragma unroll
-    for (int n = 0; n < NS; ++n) {
-      if (n < n_state) {
-        S[n] = fmaf(expf(step * A[n]), S[n], drive * B[n]);
-        y = fmaf(S[n], C[n], y);
-      }
+  const float skip = d[cc];
+  const int first = q_start[r], last = q_start[r + 1];
+  const int row = 2 * n_state;
+  for (int t0 = first; t0 < last; t0 += kScanAhead) {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();                  // the tokens before have been read by every lane
+    for (int e = threadIdx.x; e < kScanAhead * row; e += blockDim.x) {
+      const int t = min(t0 + e / row, last - 1);
+      shared_bc[e] = bc[static_cast<long>(t) * row + e % row];
     }
-    y = fmaf(skip, xv, y);
-    out[static_cast<long>(t) * channels + c] = from_float<T>(y * silu(gate));
+    float xv[kScanAhead], step[kScanAhead], gate[kScanAhead];
+#pragma unroll
+    for (int u = 0; u < kScanAhead; ++u) {
+      const long t = min(t0 + u, last - 1);
+      xv[u] = to_float(x[t * channels + cc]);
+      step[u] = dt[t * channels + cc];
+      gate[u] = to_float(z[t * z_stride + cc]);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+    for (int u = 0; u < kScanAhead; ++u) {
+      if (t0 + u >= last) break;
+      const float h = softplus(step[u]);
+      const float* B = shared_bc + u * row;
+      const float* C = B + n_state;
+      const float drive = h * xv[u];
+      float y = 0.f;
+#pragma unroll
+      for (int n = 0; n < NS; ++n) {
+        if (n < n_state) {
+          S[n] = fmaf(expf(h * A[n]), S[n], drive * B[n]);
+          y = fmaf(S[n], C[n], y);
+        }
+      }
+      y = fmaf(skip, xv[u], y);
+      if (works) out[static_cast<long>(t0 + u) * channels + c] = from_float<T>(y * silu(gate[u]));
+    }
   }
+  if (!works) return;
 #pragma unroll
   for (int n = 0; n < NS; ++n)
     if (n < n_state) kept[n] = S[n];
@@ -150,7 +178,7 @@ int akv_selective_scan(const void* x, int dtype, const float* dt, const float* b
   if (n_state <= 0 || n_state > 256) return -2;
   const dim3 grid(seqs, (channels + 63) / 64);
 #define AKV_SCAN(T, NS)                                                                                             \
-  selective_scan_kernel<T, NS><<<grid, 64, 0, stream>>>(static_cast<const T*>(x), dt, bc, static_cast<const T*>(z), \
+  selective_scan_kernel<T, NS><<<grid, 64, kScanAhead * 2 * n_state * 4, stream>>>(static_cast<const T*>(x), dt, bc, static_cast<const T*>(z), \
                                                         z_stride, a, d, state, state_stride, q_start, seq_slots,    \
                                                         static_cast<T*>(out), channels, n_state)
   AKV_DISPATCH(dtype, T, {

@@ -208,6 +208,34 @@ class PartsKernels:
             held = self.__dict__["_heads_buffer"] = torch.empty(max(need, 1 << 22), dtype=torch.bfloat16, device=self.device)
         return held[:need].view(heads, tokens, outs)
 
+    LATENT_WAVES = 1024             # steps of few tokens cut every token's keys into runs until about so many waves work
+    LATENT_MIN_RUN = 64
+    LATENT_MAX_RUNS = 64
+
+    def _latent_runs(self, tiles: int, kv_rank: int, span: int):
+        """(keys per run, runs, workspace) for a launch of `tiles` waves whose tokens see at most `span` keys: one run
+        where the tiles alone fill the device; else runs of a size that depends on the step's shape and the span's bound
+        only - a recorded step is cut as the same step run eagerly."""
+        if tiles * 2 >= self.LATENT_WAVES or span <= self.LATENT_MIN_RUN:
+            return 0, 1, None
+        wanted = max(self.LATENT_WAVES // tiles, 1)
+        segment = max((span + wanted - 1) // wanted, self.LATENT_MIN_RUN)
+        segment = (segment + 31) // 32 * 32
+        segments = (span + segment - 2) // segment + 1            # the most runs that a span of keys can touch
+        while segments > self.LATENT_MAX_RUNS:
+            segment *= 2
+            segments = (span + segment - 2) // segment + 1
+        if segments <= 1:
+            return 0, 1, None
+        need = tiles * segments * 16 * (kv_rank + 2)
+        held = self.__dict__.get("_latent_parts")
+        if held is None or held.numel() < need:
+            if torch.cuda.is_current_stream_capturing():
+                self._refuse("a recorded step needs more room for the runs' shares than the steps before it")
+            self.__dict__.setdefault("_latent_outgrown", []).append(held)
+            held = self.__dict__["_latent_parts"] = torch.empty(max(need, 1 << 22), dtype=torch.float32, device=self.device)
+        return segment, segments, held
+
     def latent_attend(self, q_abs, records, ctx, meta, heads, kv_rank, scale, window, out, latents_t=None) -> None:
         """Every head of every token attends the records [kv_rank + rot] of its request's last `window` tokens (all,
         if None): softmax((q_abs . record) * scale), then the weighted sum of the records' first kv_rank dimensions
@@ -236,11 +264,13 @@ class PartsKernels:
             if not self.latent_on_matrix_cores(heads, kv_rank, width, records.shape[2], records.dtype):
                 self._refuse("the matrix-core attention over latents does not take these sizes")
             self._dense(latents_t, "latents_t", torch.bfloat16, (records.shape[0], 1, kv_rank, records.shape[2]))
+            segment, segments, parts = self._latent_runs(tokens * heads // 16, kv_rank,
+                                                         int(window) if window is not None else ctx.max_seq_len)
             self._check(self._parts().akv_latent_attend_mfma(
                 _ptr(q_abs), _ptr(records), _ptr(latents_t), _ptr(ctx.seq_of_token), _ptr(ctx.positions),
                 _ptr(meta.block_table), _ptr(meta.rows), meta.width, _ptr(out), tokens, heads, kv_rank, width,
                 records.shape[2], _long(records.shape[0]), ctypes.c_float(scale), int(window) if window is not None else 0,
-                self._stream()), "latent_attend on the matrix cores")
+                segment, segments, _ptr(parts), self._stream()), "latent_attend on the matrix cores")
             return
         self._check(self._parts().akv_latent_attend(
             _ptr(q_abs), _ptr(records), self._code_of(records), _ptr(ctx.seq_of_token), _ptr(ctx.positions),
@@ -301,16 +331,14 @@ class PartsKernels:
             channels, n_state, self._stream()), "selective_scan")
 
     # ---- routed feed-forward -------------------------------------------------------------------------------------------
-    def route(self, x, router, gates, top: int, groups: int, keep: int) -> None:
-        """gates[t, e] = softmax(router x_t)[e] for the `top` best experts among those of the `keep` best of `groups`
+    def route(self, logits, gates, top: int, groups: int, keep: int) -> None:
+        """gates[t, e] = softmax(logits_t)[e] for the `top` best experts among those of the `keep` best of `groups`
         groups of neighbouring experts (a group's score is its best expert's), 0 for every other expert."""
-        tokens, hidden = x.shape
-        experts = router.shape[0]
-        self._dense(x, "x")
-        self._dense(router, "router", torch.float32, (experts, hidden))
+        tokens, experts = logits.shape
+        self._dense(logits, "logits", torch.float32)
         self._dense(gates, "gates", torch.float32, (tokens, experts))
-        self._check(self._parts().akv_route(_ptr(x), self._code_of(x), _ptr(router), _ptr(gates), tokens, hidden, experts,
-                                            top, groups, keep, self._stream()), "route")
+        self._check(self._parts().akv_route(_ptr(logits), _ptr(gates), tokens, experts, top, groups, keep, self._stream()),
+                    "route")
 
     def gate_relu_squared(self, up, gates, act) -> None:
         """act[t, e * ff + j] = gates[t, e] * relu(up[t, e * ff + j])^2 (may be in place)."""

@@ -40,7 +40,9 @@ class RoutedExperts(Part):
             raise ValueError(f"{self.top} experts a token cannot be chosen from {self.kept} groups of {self.experts // self.groups}")
         self.up = Linear(runtime, self.hidden, [self.ff] * self.experts, [f"e{e}.up" for e in range(self.experts)])
         self.down = Linear(runtime, self.experts * self.ff, [self.hidden], ["down"])     # (adopted at load: side by side)
-        self.router = None
+        # the router's logits are a product like any other, with float32 sums left as they are: what the file stores in
+        # 16 bits is exact in the operands, so nothing of the logits is formed in less than 32 bits
+        self.router = Linear(runtime, self.hidden, [self.experts], ["router"])
 
     def _prefix(self, prefix):
         return f"{prefix}{self.name}."
@@ -50,22 +52,24 @@ class RoutedExperts(Part):
 
     def tensors(self, prefix):
         p = self._prefix(prefix)
-        return self.up.tensors(p) + self._down_specs(p) + [TensorSpec(p + "router", (self.experts, self.hidden), MATRIX)]
+        return self.up.tensors(p) + self._down_specs(p) + self.router.tensors(p)
 
     def load(self, fetch, prefix):
         p = self._prefix(prefix)
         self.up.load(fetch, p)
         self.down.adopt(torch.cat([fetch(spec) for spec in self._down_specs(p)], dim=1).contiguous())
-        self.router = fetch(TensorSpec(p + "router", (self.experts, self.hidden), MATRIX)).to(torch.float32).contiguous()
+        self.router.load(fetch, p)
 
     def weight_bytes(self):
-        return self.up.weight_bytes() + self.down.weight_bytes() + self.experts * self.hidden * 4
+        return self.up.weight_bytes() + self.down.weight_bytes() + self.router.weight_bytes()
 
     def forward(self, x, ctx):
         k, dtype = self.rt.kernels, self.rt.dtype
         tokens = x.shape[0]
+        logits = ctx.arena.take((tokens, self.experts), torch.float32)
+        self.router.forward(x, logits)
         gates = ctx.arena.take((tokens, self.experts), torch.float32)
-        k.route(x, self.router, gates, self.top, self.groups, self.kept)
+        k.route(logits, gates, self.top, self.groups, self.kept)
         up = ctx.arena.take((tokens, self.experts * self.ff), dtype)
         self.up.forward(x, up)
         act = ctx.arena.take((tokens, self.experts * self.ff), dtype)

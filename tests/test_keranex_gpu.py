@@ -269,7 +269,8 @@ def test_latent_attention_over_records(hip, dtype, heads, kv_rank, rot, page, po
 @pytest.mark.parametrize("heads,kv_rank,rot,page", [(16, 128, 32, 16), (32, 512, 64, 16), (16, 256, 32, 8), (48, 128, 64, 32)])
 @pytest.mark.parametrize("portions,window", [([(0, 1)], 5), ([(0, 70)], 19), ([(64, 1), (17, 1), (0, 1)], 16), ([(31, 2)], 32),
                                              ([(5, 7), (63, 2), (130, 1), (0, 70)], 40), ([(200, 3), (0, 9)], None),
-                                             ([(500, 40)], 300)])
+                                             ([(500, 40)], 300), ([(1500, 1), (40, 1), (700, 1)], 1024),
+                                             ([(2100, 1), (3, 2)], None)])
 def test_latent_attention_on_the_matrix_cores(hip, heads, kv_rank, rot, page, portions, window):
     """bfloat16 queries and records; the latents a second time with the keys contiguous.  Against the plain function on
     the same rounded operands."""
@@ -379,7 +380,7 @@ def test_router_and_gated_activation(hip, dtype, experts, top, groups, keep):
     x = rand(tokens, hidden, seed=1, dtype=dtype)
     router = rand(experts, hidden, seed=2, scale=0.3)
     gates = torch.empty(tokens, experts, device="cuda")
-    hip.route(x.cuda(), router.cuda(), gates, top, groups, keep)
+    hip.route((x.float() @ router.T).cuda(), gates, top, groups, keep)
     chosen, weights = plain.route(x.float(), router, experts, top, groups, keep)
     want = torch.zeros(tokens, experts).scatter_(1, chosen, weights)
     torch.testing.assert_close(gates.cpu(), want, rtol=1e-5, atol=1e-6)

@@ -350,8 +350,8 @@ class TorchKernels(KernelSet):
                 out[t] = (y * z * torch.sigmoid(z)).to(out.dtype)
             state[slot, :channels * n_state] = S.reshape(-1)
 
-    def route(self, x, router, gates, top, groups, keep):
-        scores = (x.float() @ router.T).softmax(-1)
+    def route(self, logits, gates, top, groups, keep):
+        scores = logits.softmax(-1)
         tokens, experts = scores.shape
         best = scores.view(tokens, groups, experts // groups).amax(-1)
         allowed = torch.zeros(tokens, groups, dtype=torch.bool)
