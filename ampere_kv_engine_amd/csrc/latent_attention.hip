@@ -133,6 +133,7 @@ __global__ __launch_bounds__(256) void heads_linear_kernel(const TX* __restrict_
   float acc[kHeadTokens];
 #pragma unroll
   for (int t = 0; t < kHeadTokens; ++t) acc[t] = 0.f;
+#pragma unroll 8
   for (int i = 0; i < ins; ++i) {
     const float weight = to_float(column[static_cast<size_t>(i) * outs]);
     const float4 a = *reinterpret_cast<const float4*>(xs + i * kHeadTokens);

@@ -66,43 +66,48 @@ __global__ __launch_bounds__(256) void conv_state_update_kernel(const T* __restr
   }
 }
 
-// ---- the scan: a thread owns a channel of a request, its row of S in registers, and walks the portion's tokens ------
-// Tokens are taken kScanAhead at a time: their inputs are asked for together (a token's own arithmetic is short, and
-// one trip to memory per token would be all a long portion's time), and the wave lays the tokens' B and C, which all
-// channels share, into LDS once.
+// ---- the scan ---------------------------------------------------------------------------------------------------------
+// A channel's state is spread over LP lanes (LP: the state's size rounded up to a power of two, at most 64; a lane owns
+// states lane, lane + LP, ... - NK of them): per token a lane forms one decay and one product per state it owns, and
+// the channel's output is the sum over its lanes, which a butterfly of lane exchanges leaves in all of them.  The
+// recurrence of a state is a chain through all tokens; everything else of a token hangs off that chain, so tokens are
+// taken kScanAhead at a time: their inputs are asked for together, the block lays their B and C, which all channels
+// share, into LDS once, and the eight sums' exchanges overlap.  exp(dt A) is formed as exp2(dt (A log2 e)).
 constexpr int kScanAhead = 8;
+constexpr float kLog2e = 1.4426950408889634f;
 
-template <typename T, int NS>
-__global__ __launch_bounds__(64) void selective_scan_kernel(const T* __restrict__ x, const float* __restrict__ dt,
-                                                            const float* __restrict__ bc, const T* __restrict__ z,
-                                                            long z_stride, const float* __restrict__ a,
-                                                            const float* __restrict__ d, float* __restrict__ state,
-                                                            long state_stride, const int* __restrict__ q_start,
-                                                            const int* __restrict__ seq_slots, T* __restrict__ out,
-                                                            int channels, int n_state) {
+template <typename T, int LP, int NK>
+__global__ __launch_bounds__(256) void selective_scan_kernel(const T* __restrict__ x, const float* __restrict__ dt,
+                                                             const float* __restrict__ bc, const T* __restrict__ z,
+                                                             long z_stride, const float* __restrict__ a,
+                                                             const float* __restrict__ d, float* __restrict__ state,
+                                                             long state_stride, const int* __restrict__ q_start,
+                                                             const int* __restrict__ seq_slots, T* __restrict__ out,
+                                                             int channels, int n_state) {
   extern __shared__ float shared_bc[];                // [kScanAhead][2 * n_state]
   const int r = blockIdx.x;
-  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  const int part = threadIdx.x % LP;                  // which of the channel's lanes
+  const int c = blockIdx.y * (256 / LP) + threadIdx.x / LP;
   const bool works = c < channels;
-  const int cc = works ? c : channels - 1;            // (a lane beyond the channels keeps the wave's steps and stores nothing)
+  const int cc = works ? c : channels - 1;            // (lanes beyond the channels keep the block's steps and store nothing)
   float* kept = state + static_cast<long>(seq_slots[r]) * state_stride + static_cast<long>(cc) * n_state;
-  float S[NS], A[NS];
+  float S[NK], A[NK];
 #pragma unroll
-  for (int n = 0; n < NS; ++n) {
-    S[n] = n < n_state ? kept[n] : 0.f;
-    A[n] = n < n_state ? a[static_cast<long>(cc) * n_state + n] : 0.f;
+  for (int k = 0; k < NK; ++k) {
+    const int n = part + k * LP;
+    S[k] = n < n_state ? kept[n] : 0.f;
+    A[k] = n < n_state ? a[static_cast<long>(cc) * n_state + n] * kLog2e : 0.f;
   }
   const float skip = d[cc];
   const int first = q_start[r], last = q_start[r + 1];
   const int row = 2 * n_state;
   for (int t0 = first; t0 < last; t0 += kScanAhead) {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();                  // the tokens before have been read by every lane
+    __syncthreads();                                  // the tokens before have been read by everybody
     for (int e = threadIdx.x; e < kScanAhead * row; e += blockDim.x) {
       const int t = min(t0 + e / row, last - 1);
       shared_bc[e] = bc[static_cast<long>(t) * row + e % row];
     }
-    float xv[kScanAhead], step[kScanAhead], gate[kScanAhead];
+    float xv[kScanAhead], step[kScanAhead], gate[kScanAhead], y[kScanAhead];
 #pragma unroll
     for (int u = 0; u < kScanAhead; ++u) {
       const long t = min(t0 + u, last - 1);
@@ -110,32 +115,55 @@ __global__ __launch_bounds__(64) void selective_scan_kernel(const T* __restrict_
       step[u] = dt[t * channels + cc];
       gate[u] = to_float(z[t * z_stride + cc]);
     }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    __syncthreads();
 #pragma unroll
     for (int u = 0; u < kScanAhead; ++u) {
-      if (t0 + u >= last) break;
       const float h = softplus(step[u]);
+      const float drive = h * xv[u];
       const float* B = shared_bc + u * row;
       const float* C = B + n_state;
-      const float drive = h * xv[u];
-      float y = 0.f;
+      float sum = 0.f;
+      if (t0 + u < last) {                            // (uniform over the block)
 #pragma unroll
-      for (int n = 0; n < NS; ++n) {
-        if (n < n_state) {
-          S[n] = fmaf(expf(h * A[n]), S[n], drive * B[n]);
-          y = fmaf(S[n], C[n], y);
+        for (int k = 0; k < NK; ++k) {
+          const int n = part + k * LP;
+          if (n < n_state) {
+            S[k] = fmaf(__builtin_amdgcn_exp2f(h * A[k]), S[k], drive * B[n]);
+            sum = fmaf(S[k], C[n], sum);
+          }
         }
       }
-      y = fmaf(skip, xv[u], y);
-      if (works) out[static_cast<long>(t0 + u) * channels + c] = from_float<T>(y * silu(gate[u]));
+      y[u] = sum;
+    }
+#pragma unroll
+    for (int offset = LP / 2; offset > 0; offset >>= 1)
+#pragma unroll
+      for (int u = 0; u < kScanAhead; ++u) y[u] += __shfl_xor(y[u], offset, kWave);
+    if (works && part < kScanAhead && t0 + part < last) {      // lane u of a channel stores token u
+      float mine = 0.f, xm = 0.f, gm = 0.f;
+#pragma unroll
+      for (int u = 0; u < kScanAhead; ++u)
+        if (u == part) {
+          mine = y[u];
+          xm = xv[u];
+          gm = gate[u];
+        }
+      out[static_cast<long>(t0 + part) * channels + c] = from_float<T>(fmaf(skip, xm, mine) * silu(gm));
+    }
+    if constexpr (LP < kScanAhead) {                  // fewer lanes than tokens: lane 0 stores the rest
+      if (works && part == 0) {
+#pragma unroll
+        for (int u = LP; u < kScanAhead; ++u)
+          if (t0 + u < last) out[static_cast<long>(t0 + u) * channels + c] = from_float<T>(fmaf(skip, xv[u], y[u]) * silu(gate[u]));
+      }
     }
   }
   if (!works) return;
 #pragma unroll
-  for (int n = 0; n < NS; ++n)
-    if (n < n_state) kept[n] = S[n];
+  for (int k = 0; k < NK; ++k) {
+    const int n = part + k * LP;
+    if (n < n_state) kept[n] = S[k];
+  }
 }
 
 }  // namespace
@@ -176,18 +204,23 @@ int akv_selective_scan(const void* x, int dtype, const float* dt, const float* b
                        const int* seq_slots, void* out, int seqs, int channels, int n_state, hipStream_t stream) {
   if (seqs <= 0) return 0;
   if (n_state <= 0 || n_state > 256) return -2;
-  const dim3 grid(seqs, (channels + 63) / 64);
-#define AKV_SCAN(T, NS)                                                                                             \
-  selective_scan_kernel<T, NS><<<grid, 64, kScanAhead * 2 * n_state * 4, stream>>>(static_cast<const T*>(x), dt, bc, static_cast<const T*>(z), \
-                                                        z_stride, a, d, state, state_stride, q_start, seq_slots,    \
-                                                        static_cast<T*>(out), channels, n_state)
+  int lanes = 1;
+  while (lanes < n_state && lanes < 64) lanes <<= 1;
+  const dim3 grid(seqs, (channels + 256 / lanes - 1) / (256 / lanes));
+#define AKV_SCAN(T, LP, NK)                                                                                         \
+  selective_scan_kernel<T, LP, NK><<<grid, 256, kScanAhead * 2 * n_state * 4, stream>>>(                              \
+      static_cast<const T*>(x), dt, bc, static_cast<const T*>(z), z_stride, a, d, state, state_stride, q_start,     \
+      seq_slots, static_cast<T*>(out), channels, n_state)
   AKV_DISPATCH(dtype, T, {
-    if (n_state <= 8) AKV_SCAN(T, 8);
-    else if (n_state <= 16) AKV_SCAN(T, 16);
-    else if (n_state <= 32) AKV_SCAN(T, 32);
-    else if (n_state <= 64) AKV_SCAN(T, 64);
-    else if (n_state <= 128) AKV_SCAN(T, 128);
-    else AKV_SCAN(T, 256);
+    if (lanes == 1) AKV_SCAN(T, 1, 1);
+    else if (lanes == 2) AKV_SCAN(T, 2, 1);
+    else if (lanes == 4) AKV_SCAN(T, 4, 1);
+    else if (lanes == 8) AKV_SCAN(T, 8, 1);
+    else if (lanes == 16) AKV_SCAN(T, 16, 1);
+    else if (lanes == 32) AKV_SCAN(T, 32, 1);
+    else if (n_state <= 64) AKV_SCAN(T, 64, 1);
+    else if (n_state <= 128) AKV_SCAN(T, 64, 2);
+    else AKV_SCAN(T, 64, 4);
   });
 #undef AKV_SCAN
   return AKV_LAUNCH_STATUS();
