@@ -113,28 +113,32 @@ __global__ void rotate_queries_kernel(const T* __restrict__ q, long tokens, int 
 // batch.
 constexpr int kHeadTokens = 8;
 
-template <typename TX, typename TW, typename TY>
+// With few tokens (SPLIT) a head's matrix is the work: a block is 64 outputs, and its four waves take every fourth
+// input each and add their sums through LDS in the waves' order.
+template <typename TX, typename TW, typename TY, bool SPLIT>
 __global__ __launch_bounds__(256) void heads_linear_kernel(const TX* __restrict__ x, long x_token_stride,
                                                            long x_head_stride, const TW* __restrict__ w,
                                                            TY* __restrict__ y, long y_token_stride, long y_head_stride,
                                                            int tokens, int ins, int outs) {
-  extern __shared__ float xs[];      // [ins][kHeadTokens]
+  extern __shared__ float xs[];      // [ins][kHeadTokens], then (SPLIT) [3][64][kHeadTokens]
   const int h = blockIdx.y;
   const int first = blockIdx.x * kHeadTokens;
-  const int j = blockIdx.z * blockDim.x + threadIdx.x;
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
+  const int j = SPLIT ? blockIdx.z * kWave + lane : blockIdx.z * blockDim.x + threadIdx.x;
   for (int e = threadIdx.x; e < ins * kHeadTokens; e += blockDim.x) {
     const int t = e / ins, i = e % ins;             // (consecutive threads read consecutive inputs of one token)
     const int n = first + t;
     xs[i * kHeadTokens + t] = n < tokens ? to_float(x[n * x_token_stride + h * x_head_stride + i]) : 0.f;
   }
   __syncthreads();
-  if (j >= outs) return;
-  const TW* column = w + static_cast<size_t>(h) * ins * outs + j;
+  const int jj = min(j, outs - 1);                  // (a thread beyond the outputs keeps the block's steps, stores nothing)
+  const TW* column = w + static_cast<size_t>(h) * ins * outs + jj;
   float acc[kHeadTokens];
 #pragma unroll
   for (int t = 0; t < kHeadTokens; ++t) acc[t] = 0.f;
+  const int begin = SPLIT ? wave : 0, stride = SPLIT ? 4 : 1;
 #pragma unroll 8
-  for (int i = 0; i < ins; ++i) {
+  for (int i = begin; i < ins; i += stride) {
     const float weight = to_float(column[static_cast<size_t>(i) * outs]);
     const float4 a = *reinterpret_cast<const float4*>(xs + i * kHeadTokens);
     const float4 b = *reinterpret_cast<const float4*>(xs + i * kHeadTokens + 4);
@@ -147,6 +151,20 @@ __global__ __launch_bounds__(256) void heads_linear_kernel(const TX* __restrict_
     acc[6] = fmaf(b.z, weight, acc[6]);
     acc[7] = fmaf(b.w, weight, acc[7]);
   }
+  if constexpr (SPLIT) {
+    float* shares = xs + ins * kHeadTokens;         // [3][64][kHeadTokens]
+    if (wave > 0) {
+#pragma unroll
+      for (int t = 0; t < kHeadTokens; ++t) shares[((wave - 1) * kWave + lane) * kHeadTokens + t] = acc[t];
+    }
+    __syncthreads();
+    if (wave > 0) return;
+#pragma unroll
+    for (int other = 0; other < 3; ++other)
+#pragma unroll
+      for (int t = 0; t < kHeadTokens; ++t) acc[t] += shares[(other * kWave + lane) * kHeadTokens + t];
+  }
+  if (j >= outs) return;
 #pragma unroll
   for (int t = 0; t < kHeadTokens; ++t) {
     const int n = first + t;
@@ -563,21 +581,30 @@ int akv_heads_linear(const void* x, int x_dtype, long x_token_stride, long x_hea
                      int outs, hipStream_t stream) {
   if (tokens <= 0 || heads <= 0) return 0;
   if (ins <= 0 || outs <= 0) return -2;
-  const size_t lds_bytes = static_cast<size_t>(ins) * kHeadTokens * 4;
+  // few tokens: blocks of 64 outputs whose waves share the inputs (not in float32, whose sums keep one order whatever
+  // the batch)
+  const bool split = tokens <= 2 * kHeadTokens && !(x_dtype == kF32 && w_dtype == kF32 && y_dtype == kF32);
+  const size_t lds_bytes = static_cast<size_t>(ins) * kHeadTokens * 4 + (split ? 3 * kWave * kHeadTokens * 4 : 0);
   if (lds_bytes > 64 * 1024) return -2;
-  // few tokens: a head's matrix is the work, cut over more blocks (a wave each); many: blocks of up to four waves
-  const int threads = tokens <= 2 * kHeadTokens ? kWave : outs >= 256 ? 256 : (outs + kWave - 1) / kWave * kWave;
-  const dim3 grid((tokens + kHeadTokens - 1) / kHeadTokens, heads, (outs + threads - 1) / threads);
-#define AKV_HEADS(TX, TW, TY)                                                                                       \
-  heads_linear_kernel<TX, TW, TY><<<grid, threads, lds_bytes, stream>>>(                                            \
+  const int threads = split ? 256 : outs >= 256 ? 256 : (outs + kWave - 1) / kWave * kWave;
+  const int per_block = split ? kWave : threads;
+  const dim3 grid((tokens + kHeadTokens - 1) / kHeadTokens, heads, (outs + per_block - 1) / per_block);
+#define AKV_HEADS_AS(TX, TW, TY, SPLIT)                                                                             \
+  heads_linear_kernel<TX, TW, TY, SPLIT><<<grid, threads, lds_bytes, stream>>>(                                     \
       static_cast<const TX*>(x), x_token_stride, x_head_stride, static_cast<const TW*>(w), static_cast<TY*>(y),    \
       y_token_stride, y_head_stride, tokens, ins, outs)
+#define AKV_HEADS(TX, TW, TY)                 \
+  do {                                        \
+    if (split) AKV_HEADS_AS(TX, TW, TY, true); \
+    else AKV_HEADS_AS(TX, TW, TY, false);     \
+  } while (0)
   if (x_dtype == kF32 && w_dtype == kF32 && y_dtype == kF32) AKV_HEADS(float, float, float);
   else if (x_dtype == kBF16 && w_dtype == kBF16 && y_dtype == kF32) AKV_HEADS(bf16_t, bf16_t, float);
   else if (x_dtype == kF32 && w_dtype == kBF16 && y_dtype == kBF16) AKV_HEADS(float, bf16_t, bf16_t);
   else if (x_dtype == kF32 && w_dtype == kBF16 && y_dtype == kF32) AKV_HEADS(float, bf16_t, float);
   else if (x_dtype == kBF16 && w_dtype == kBF16 && y_dtype == kBF16) AKV_HEADS(bf16_t, bf16_t, bf16_t);
   else return -1;
+#undef AKV_HEADS_AS
 #undef AKV_HEADS
   return AKV_LAUNCH_STATUS();
 }

@@ -84,7 +84,7 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(const T* __restrict
                                                              long state_stride, const int* __restrict__ q_start,
                                                              const int* __restrict__ seq_slots, T* __restrict__ out,
                                                              int channels, int n_state) {
-  extern __shared__ float shared_bc[];                // [kScanAhead][2 * n_state]
+  extern __shared__ float shared_bc[];                // two of [kScanAhead][2 * n_state]
   const int r = blockIdx.x;
   const int part = threadIdx.x % LP;                  // which of the channel's lanes
   const int c = blockIdx.y * (256 / LP) + threadIdx.x / LP;
@@ -101,26 +101,40 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(const T* __restrict
   const float skip = d[cc];
   const int first = q_start[r], last = q_start[r + 1];
   const int row = 2 * n_state;
-  for (int t0 = first; t0 < last; t0 += kScanAhead) {
-    __syncthreads();                                  // the tokens before have been read by everybody
+  // the tokens after these are asked for while these are worked on: their inputs into a second set of registers, their
+  // B and C into the other half of the LDS buffer
+  float xn[kScanAhead], stepn[kScanAhead], gaten[kScanAhead];
+  auto fetch = [&](int t0, float* into) {
     for (int e = threadIdx.x; e < kScanAhead * row; e += blockDim.x) {
       const int t = min(t0 + e / row, last - 1);
-      shared_bc[e] = bc[static_cast<long>(t) * row + e % row];
+      into[e] = bc[static_cast<long>(t) * row + e % row];
     }
-    float xv[kScanAhead], step[kScanAhead], gate[kScanAhead], y[kScanAhead];
 #pragma unroll
     for (int u = 0; u < kScanAhead; ++u) {
       const long t = min(t0 + u, last - 1);
-      xv[u] = to_float(x[t * channels + cc]);
-      step[u] = dt[t * channels + cc];
-      gate[u] = to_float(z[t * z_stride + cc]);
+      xn[u] = to_float(x[t * channels + cc]);
+      stepn[u] = dt[t * channels + cc];
+      gaten[u] = to_float(z[t * z_stride + cc]);
     }
-    __syncthreads();
+  };
+  if (first < last) fetch(first, shared_bc);
+  int turn = 0;
+  for (int t0 = first; t0 < last; t0 += kScanAhead, turn ^= 1) {
+    float xv[kScanAhead], step[kScanAhead], gate[kScanAhead], y[kScanAhead];
+#pragma unroll
+    for (int u = 0; u < kScanAhead; ++u) {
+      xv[u] = xn[u];
+      step[u] = stepn[u];
+      gate[u] = gaten[u];
+    }
+    __syncthreads();                                  // this turn's B and C are in place; the other half has been read
+    const float* mine_bc = shared_bc + turn * kScanAhead * row;
+    if (t0 + kScanAhead < last) fetch(t0 + kScanAhead, shared_bc + (turn ^ 1) * kScanAhead * row);
 #pragma unroll
     for (int u = 0; u < kScanAhead; ++u) {
       const float h = softplus(step[u]);
       const float drive = h * xv[u];
-      const float* B = shared_bc + u * row;
+      const float* B = mine_bc + u * row;
       const float* C = B + n_state;
       float sum = 0.f;
       if (t0 + u < last) {                            // (uniform over the block)
@@ -208,7 +222,7 @@ int akv_selective_scan(const void* x, int dtype, const float* dt, const float* b
   while (lanes < n_state && lanes < 64) lanes <<= 1;
   const dim3 grid(seqs, (channels + 256 / lanes - 1) / (256 / lanes));
 #define AKV_SCAN(T, LP, NK)                                                                                         \
-  selective_scan_kernel<T, LP, NK><<<grid, 256, kScanAhead * 2 * n_state * 4, stream>>>(                              \
+  selective_scan_kernel<T, LP, NK><<<grid, 256, 2 * kScanAhead * 2 * n_state * 4, stream>>>(                              \
       static_cast<const T*>(x), dt, bc, static_cast<const T*>(z), z_stride, a, d, state, state_stride, q_start,     \
       seq_slots, static_cast<T*>(out), channels, n_state)
   AKV_DISPATCH(dtype, T, {

@@ -54,8 +54,79 @@ __global__ void note_fed_tokens_kernel(const int* __restrict__ ids, const int* _
 }
 
 // ---- stream += norm_post(delta); out = norm_pre(stream) -----------------------------------------------------------------
-// One block per row, three passes over a row that the caches hold: the branch's sum of squares; the update of the
-// residual sum, which gathers the new sum of squares as it goes; the normed row.
+// One block per row.  Rows of up to 256 * 4 * GROUPS elements (a multiple of 4) stay in registers from their one trip to
+// memory to the store; others take three passes over a row that the caches hold: the branch's sum of squares; the
+// update of the residual sum, which gathers the new sum of squares as it goes; the normed row.
+template <typename T> __device__ __forceinline__ float4 read4(const T* p);
+template <> __device__ __forceinline__ float4 read4<float>(const float* p) { return *reinterpret_cast<const float4*>(p); }
+template <> __device__ __forceinline__ float4 read4<bf16_t>(const bf16_t* p) {
+  const uint2 v = *reinterpret_cast<const uint2*>(p);
+  return make_float4(__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xffff0000u), __uint_as_float(v.y << 16),
+                     __uint_as_float(v.y & 0xffff0000u));
+}
+template <typename T> __device__ __forceinline__ void write4(T* p, float4 v);
+template <> __device__ __forceinline__ void write4<float>(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+template <> __device__ __forceinline__ void write4<bf16_t>(bf16_t* p, float4 v) {
+  uint2 packed;
+  packed.x = bf16_pair(v.x, v.y);
+  packed.y = bf16_pair(v.z, v.w);
+  *reinterpret_cast<uint2*>(p) = packed;
+}
+
+template <typename T, int GROUPS>
+__global__ __launch_bounds__(256) void norm_add_norm_rows_kernel(float* __restrict__ stream, const T* __restrict__ delta,
+                                                                 const float* __restrict__ post_weight, float post_eps,
+                                                                 const float* __restrict__ pre_weight, float pre_eps,
+                                                                 T* __restrict__ out, int hidden) {
+  __shared__ float scratch[16];
+  const size_t base = static_cast<size_t>(blockIdx.x) * hidden;
+  float4 kept[GROUPS], added[GROUPS];
+  // every load goes out before anything waits (a group beyond the row reads its last four values and counts for nothing)
+#pragma unroll
+  for (int j = 0; j < GROUPS; ++j) {
+    const int i = min((j * 256 + static_cast<int>(threadIdx.x)) * 4, hidden - 4);
+    kept[j] = read4<float>(stream + base + i);
+    if (delta != nullptr) added[j] = read4<T>(delta + base + i);
+  }
+  float squares = 0.f;
+  if (delta != nullptr) {
+    float post_scale = 1.f;
+    if (post_weight != nullptr) {
+      float acc = 0.f;
+#pragma unroll
+      for (int j = 0; j < GROUPS; ++j)
+        if ((j * 256 + static_cast<int>(threadIdx.x)) * 4 < hidden)
+          acc += added[j].x * added[j].x + added[j].y * added[j].y + added[j].z * added[j].z + added[j].w * added[j].w;
+      post_scale = rsqrtf(block_sum(acc, scratch) / static_cast<float>(hidden) + post_eps);
+    }
+#pragma unroll
+    for (int j = 0; j < GROUPS; ++j) {
+      const int i = (j * 256 + static_cast<int>(threadIdx.x)) * 4;
+      if (i >= hidden) continue;
+      float4 d = added[j];
+      if (post_weight != nullptr) {
+        const float4 w = read4<float>(post_weight + i);
+        d = make_float4(d.x * post_scale * w.x, d.y * post_scale * w.y, d.z * post_scale * w.z, d.w * post_scale * w.w);
+      }
+      kept[j] = make_float4(kept[j].x + d.x, kept[j].y + d.y, kept[j].z + d.z, kept[j].w + d.w);
+      write4<float>(stream + base + i, kept[j]);
+    }
+  }
+  if (out == nullptr) return;
+#pragma unroll
+  for (int j = 0; j < GROUPS; ++j)
+    if ((j * 256 + static_cast<int>(threadIdx.x)) * 4 < hidden)
+      squares += kept[j].x * kept[j].x + kept[j].y * kept[j].y + kept[j].z * kept[j].z + kept[j].w * kept[j].w;
+  const float scale = rsqrtf(block_sum(squares, scratch) / static_cast<float>(hidden) + pre_eps);
+#pragma unroll
+  for (int j = 0; j < GROUPS; ++j) {
+    const int i = (j * 256 + static_cast<int>(threadIdx.x)) * 4;
+    if (i >= hidden) continue;
+    const float4 w = read4<float>(pre_weight + i), v = kept[j];
+    write4<T>(out + base + i, make_float4(v.x * scale * w.x, v.y * scale * w.y, v.z * scale * w.z, v.w * scale * w.w));
+  }
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void norm_add_norm_kernel(float* __restrict__ stream, const T* __restrict__ delta,
                                                             const float* __restrict__ post_weight, float post_eps,
@@ -129,9 +200,13 @@ int akv_norm_add_norm(float* stream_buf, const void* delta, const float* post_we
                       hipStream_t stream) {
   if (tokens <= 0) return 0;
   if (out != nullptr && pre_weight == nullptr) return -2;
-  AKV_DISPATCH(dtype, T, norm_add_norm_kernel<T><<<tokens, 256, 0, stream>>>(
-                             stream_buf, static_cast<const T*>(delta), post_weight, post_eps, pre_weight, pre_eps,
-                             static_cast<T*>(out), hidden));
+#define AKV_NORM_ARGS stream_buf, static_cast<const T*>(delta), post_weight, post_eps, pre_weight, pre_eps, static_cast<T*>(out), hidden
+  AKV_DISPATCH(dtype, T, {
+    if (hidden % 4 == 0 && hidden >= 4 && hidden <= 256 * 4 * 2) norm_add_norm_rows_kernel<T, 2><<<tokens, 256, 0, stream>>>(AKV_NORM_ARGS);
+    else if (hidden % 4 == 0 && hidden <= 256 * 4 * 8) norm_add_norm_rows_kernel<T, 8><<<tokens, 256, 0, stream>>>(AKV_NORM_ARGS);
+    else norm_add_norm_kernel<T><<<tokens, 256, 0, stream>>>(AKV_NORM_ARGS);
+  });
+#undef AKV_NORM_ARGS
   return AKV_LAUNCH_STATUS();
 }
 }

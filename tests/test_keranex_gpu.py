@@ -153,7 +153,7 @@ def test_pair_embedding_across_steps(hip, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("hidden", [24, 257, 1024])
+@pytest.mark.parametrize("hidden", [24, 257, 1024, 4100])
 def test_norm_after_add_and_norm_before(hip, dtype, hidden):
     stream, delta = rand(5, hidden, seed=1), rand(5, hidden, seed=2, scale=3.0, dtype=dtype)
     post, pre = 1 + rand(hidden, seed=3, scale=0.1), 1 + rand(hidden, seed=4, scale=0.1)
@@ -216,9 +216,12 @@ def test_products_per_head(hip, x_dtype, w_dtype, y_dtype, tokens, heads, ins, o
     want = torch.einsum("thi,hio->tho", x[..., :ins].float(), w.float())
     torch.testing.assert_close(y[..., :outs].cpu().float(), want, **tol(y_dtype))
     assert (y[..., outs:] == 7.0).all()
-    one = torch.empty(1, heads, outs + 3, dtype=y_dtype, device="cuda")        # a token's sums do not depend on its batch
+    one = torch.empty(1, heads, outs + 3, dtype=y_dtype, device="cuda")        # a token's sums do not depend on its batch:
     hip.heads_linear(x[tokens - 1:].contiguous().cuda(), ins + 5, w.cuda(), one, outs + 3)
-    assert torch.equal(one[..., :outs], y[tokens - 1:, :, :outs])
+    if x_dtype == w_dtype == y_dtype == torch.float32:                         # in float32 not by a bit
+        assert torch.equal(one[..., :outs], y[tokens - 1:, :, :outs])
+    else:
+        torch.testing.assert_close(one[..., :outs].float(), y[tokens - 1:, :, :outs].float(), **tol(y_dtype))
 
 
 def records_case(dtype, kv_rank, rot, page, portions, window, seed):
