@@ -64,10 +64,12 @@ int akv_conv_silu(const void* x, long x_stride, int dtype, const void* weight, c
 int akv_conv_state_update(const void* x, long x_stride, int dtype, float* state, long state_stride, long conv_at,
                           const int* q_start, const int* seq_slots, int seqs, int channels, int taps,
                           hipStream_t stream);
-// S [channels, n_state] at the start of a slot's state; dt (before softplus), bc = [B | C] float32
-int akv_selective_scan(const void* x, int dtype, const float* dt, const float* bc, const void* z, long z_stride,
+// S [channels, n_state] at the start of a slot's state; dt [tokens, channels] (before softplus, which is taken in
+// place), bc = [B | C] float32
+int akv_selective_scan(const void* x, int dtype, float* dt, const float* bc, const void* z, long z_stride,
                        const float* a, const float* d, float* state, long state_stride, const int* q_start,
-                       const int* seq_slots, void* out, int seqs, int channels, int n_state, hipStream_t stream);
+                       const int* seq_slots, void* out, int tokens, int seqs, int channels, int n_state,
+                       hipStream_t stream);
 
 // ---- routed feed-forward (routed.hip) -------------------------------------------------------------------------------
 // logits [tokens, experts] float32 -> gates [tokens, experts] float32: the softmax score of the chosen experts, 0 elsewhere

@@ -88,6 +88,30 @@ __global__ void gate_relu_squared_kernel(const T* __restrict__ up, const float* 
   act[index] = from_float<T>(value);
 }
 
+// The same, eight values a thread (16 bytes of bfloat16 in, 16 out) where an expert's width is a multiple of 8.
+__global__ void gate_relu_squared_by8_kernel(const bf16_t* __restrict__ up, const float* __restrict__ gates,
+                                             bf16_t* __restrict__ act, long tokens, int experts, int ff) {
+  const long index = (static_cast<long>(blockIdx.x) * blockDim.x + threadIdx.x) * 8;
+  const long width = static_cast<long>(experts) * ff;
+  if (index >= tokens * width) return;
+  const long n = index / width;
+  const int e = static_cast<int>((index % width) / ff);
+  const float g = gates[n * experts + e];
+  uint4 packed = make_uint4(0u, 0u, 0u, 0u);
+  if (g != 0.f) {
+    const uint4 raw = *reinterpret_cast<const uint4*>(up + index);
+    const uint32_t words[4] = {raw.x, raw.y, raw.z, raw.w};
+    uint32_t outs[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const float lo = fmaxf(__uint_as_float(words[k] << 16), 0.f), hi = fmaxf(__uint_as_float(words[k] & 0xffff0000u), 0.f);
+      outs[k] = bf16_pair(g * (lo * lo), g * (hi * hi));
+    }
+    packed = make_uint4(outs[0], outs[1], outs[2], outs[3]);
+  }
+  *reinterpret_cast<uint4*>(act + index) = packed;
+}
+
 }  // namespace
 
 extern "C" {
@@ -108,6 +132,11 @@ int akv_gate_relu_squared(const void* up, const float* gates, void* act, int dty
                           hipStream_t stream) {
   const long count = tokens * experts * ff;
   if (count <= 0) return 0;
+  if (dtype == kBF16 && ff % 8 == 0) {
+    gate_relu_squared_by8_kernel<<<static_cast<unsigned>((count / 8 + 255) / 256), 256, 0, stream>>>(
+        static_cast<const bf16_t*>(up), gates, static_cast<bf16_t*>(act), tokens, experts, ff);
+    return AKV_LAUNCH_STATUS();
+  }
   AKV_DISPATCH(dtype, T, gate_relu_squared_kernel<T><<<static_cast<unsigned>((count + 255) / 256), 256, 0, stream>>>(
                              static_cast<const T*>(up), gates, static_cast<T*>(act), tokens, experts, ff));
   return AKV_LAUNCH_STATUS();

@@ -66,6 +66,12 @@ __global__ __launch_bounds__(256) void conv_state_update_kernel(const T* __restr
   }
 }
 
+// ---- step sizes: dt <- softplus(dt), every element for itself (inside the scan each of a channel's lanes would repeat it) --
+__global__ void softplus_kernel(float* __restrict__ values, long count) {
+  const long i = static_cast<long>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < count) values[i] = softplus(values[i]);
+}
+
 // ---- the scan ---------------------------------------------------------------------------------------------------------
 // A channel's state is spread over LP lanes (LP: the state's size rounded up to a power of two, at most 64; a lane owns
 // states lane, lane + LP, ... - NK of them): per token a lane forms one decay and one product per state it owns, and
@@ -132,7 +138,7 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(const T* __restrict
     if (t0 + kScanAhead < last) fetch(t0 + kScanAhead, shared_bc + (turn ^ 1) * kScanAhead * row);
 #pragma unroll
     for (int u = 0; u < kScanAhead; ++u) {
-      const float h = softplus(step[u]);
+      const float h = step[u];                        // (softplus has been taken)
       const float drive = h * xv[u];
       const float* B = mine_bc + u * row;
       const float* C = B + n_state;
@@ -213,11 +219,16 @@ int akv_conv_state_update(const void* x, long x_stride, int dtype, float* state,
   return AKV_LAUNCH_STATUS();
 }
 
-int akv_selective_scan(const void* x, int dtype, const float* dt, const float* bc, const void* z, long z_stride,
+int akv_selective_scan(const void* x, int dtype, float* dt, const float* bc, const void* z, long z_stride,
                        const float* a, const float* d, float* state, long state_stride, const int* q_start,
-                       const int* seq_slots, void* out, int seqs, int channels, int n_state, hipStream_t stream) {
+                       const int* seq_slots, void* out, int tokens, int seqs, int channels, int n_state,
+                       hipStream_t stream) {
   if (seqs <= 0) return 0;
   if (n_state <= 0 || n_state > 256) return -2;
+  if (tokens > 0) {
+    const long count = static_cast<long>(tokens) * channels;
+    softplus_kernel<<<static_cast<unsigned>((count + 255) / 256), 256, 0, stream>>>(dt, count);
+  }
   int lanes = 1;
   while (lanes < n_state && lanes < 64) lanes <<= 1;
   const dim3 grid(seqs, (channels + 256 / lanes - 1) / (256 / lanes));

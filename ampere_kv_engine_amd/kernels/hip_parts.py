@@ -312,7 +312,7 @@ class PartsKernels:
     def selective_scan(self, x, dt, bc, xz, a, d, state, taps, ctx, out) -> None:
         """Per request and channel, token after token: S <- exp(softplus(dt) A) S + softplus(dt) x B, y = S C + D x,
         out = y * silu(z), with z the second half of `xz`'s columns and S [channels, n_state] at the start of the
-        request's state (read at the portion's start, written back at its end)."""
+        request's state (read at the portion's start, written back at its end).  `dt` is left as softplus(dt)."""
         tokens, channels = x.shape
         n_state = a.shape[1]
         self._dense(x, "x", None, (tokens, channels))
@@ -327,8 +327,8 @@ class PartsKernels:
         z = xz[:, channels:]
         self._check(self._parts().akv_selective_scan(
             _ptr(x), self._code_of(x), _ptr(dt), _ptr(bc), ctypes.c_void_p(z.data_ptr()), _long(2 * channels), _ptr(a),
-            _ptr(d), _ptr(state), _long(state.shape[1]), _ptr(ctx.q_start), _ptr(ctx.seq_slots), _ptr(out), ctx.num_seqs,
-            channels, n_state, self._stream()), "selective_scan")
+            _ptr(d), _ptr(state), _long(state.shape[1]), _ptr(ctx.q_start), _ptr(ctx.seq_slots), _ptr(out), tokens,
+            ctx.num_seqs, channels, n_state, self._stream()), "selective_scan")
 
     # ---- routed feed-forward -------------------------------------------------------------------------------------------
     def route(self, logits, gates, top: int, groups: int, keep: int) -> None:

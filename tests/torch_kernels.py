@@ -338,11 +338,12 @@ class TorchKernels(KernelSet):
 
     def selective_scan(self, x, dt, bc, xz, a, d, state, taps, ctx, out):
         channels, n_state = a.shape
+        dt.copy_(torch.nn.functional.softplus(dt, threshold=20.0))          # (taken in place, as the kernel does)
         for r in range(ctx.num_seqs):
             first, last, slot = ctx.host_q_start[r], ctx.host_q_start[r + 1], ctx.host_seq_slots[r]
             S = state[slot, :channels * n_state].view(channels, n_state).clone()
             for t in range(first, last):
-                step = torch.nn.functional.softplus(dt[t], threshold=20.0)
+                step = dt[t]
                 xv = x[t].float()
                 S = torch.exp(step[:, None] * a) * S + (step * xv)[:, None] * bc[t, None, :n_state]
                 y = S @ bc[t, n_state:] + d * xv
