@@ -277,8 +277,8 @@ def read_prompts(args, folder: str) -> list[list[int]]:
             raise SystemExit(f"{args.prompts_file} holds no prompt")
         return prompts
     if args.prompt_len is not None:
-        with open(f"{folder}/config.json") as handle:
-            vocab = json.load(handle)["vocab_size"]
+        from .config.registry import load_config
+        vocab = load_config(folder).to_model_spec().vocab_size      # (every architecture names it in keys of its own)
         generator = torch.Generator().manual_seed(args.prompt_seed)
         return [torch.randint(0, vocab, (args.prompt_len,), generator=generator).tolist()]
     if args.prompt_ids is not None:
