@@ -37,7 +37,7 @@ KERANEX_B = dict(
     embedding=dict(bigram=dict(buckets=1, mul_prev=1, mul_cur=1)),
     layers=[
         dict(type="latent_attention", mixer=LATENT(12, 32, 16, 32, 72, 40, 19, 0.15, 10000.0), mlp=MOE(2, 2, 2, 2, 32)),
-        dict(type="mamba1", mixer=SCAN(128, 24, 4, 2), mlp=MOE(8, 2, 2, 1, 8)),
+        dict(type="mamba1", mixer=SCAN(128, 20, 4, 2), mlp=MOE(8, 2, 2, 1, 8)),
         dict(type="latent_attention", mixer=LATENT(2, 16, 4, 8, 24, 8, 1, 0.25, 50.0), mlp=None),
         dict(type="latent_attention", mixer=LATENT(4, 16, 16, 16, 72, 32, 19, 0.25, 10000.0, kv_from=0), mlp=MOE(3, 1, 3, 1, 40)),
     ])
@@ -47,7 +47,7 @@ KERANEX_C = dict(
     architecture="Keranex", vocab=300, width=128, norm=dict(eps=1e-5),
     embedding=dict(bigram=dict(buckets=64, mul_prev=7, mul_cur=9)),
     layers=[
-        dict(type="latent_attention", mixer=LATENT(16, 32, 32, 32, 128, 64, 40, 0.12, 10000.0), mlp=MOE(4, 2, 2, 1, 32)),
+        dict(type="latent_attention", mixer=LATENT(16, 32, 32, 32, 128, 64, 36, 0.12, 10000.0), mlp=MOE(4, 2, 2, 1, 32)),
         dict(type="mamba1", mixer=SCAN(128, 8, 8, 4), mlp=None),
         dict(type="latent_attention", mixer=LATENT(32, 16, 32, 16, 128, 48, 24, 0.15, 10000.0, kv_from=0), mlp=MOE(4, 2, 2, 1, 32)),
     ])

@@ -201,7 +201,7 @@ def test_norm_after_add_and_norm_before(hip, dtype, hidden):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("q_rank,kv_rank,rot,rot_dims,page", [(24, 40, 8, 8, 4), (80, 128, 32, 32, 16), (16, 72, 12, 6, 8)])
+@pytest.mark.parametrize("q_rank,kv_rank,rot,rot_dims,page", [(24, 40, 8, 8, 4), (96, 192, 64, 64, 16), (16, 72, 12, 6, 8)])
 def test_latent_encode_and_rotated_queries(hip, dtype, q_rank, kv_rank, rot, rot_dims, page):
     tokens, heads, dim, base = 11, 3, 16, 100.0
     down = rand(tokens, q_rank + kv_rank + rot, seed=1, dtype=dtype)
@@ -281,7 +281,7 @@ def records_case(dtype, kv_rank, rot, page, portions, window, seed):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("heads,kv_rank,rot,page", [(3, 40, 8, 4), (8, 128, 32, 16), (12, 72, 16, 8), (2, 300, 64, 16), (1, 520, 64, 32)])
+@pytest.mark.parametrize("heads,kv_rank,rot,page", [(3, 40, 8, 4), (8, 192, 64, 16), (12, 72, 16, 8), (2, 300, 64, 16), (1, 520, 64, 32)])
 @pytest.mark.parametrize("portions,window", [([(0, 1)], 5), ([(0, 70)], 19), ([(64, 1), (17, 1), (0, 1)], 16),
                                              ([(5, 7), (63, 2), (130, 1), (0, 70)], 40), ([(200, 3), (0, 9)], None)])
 def test_latent_attention_over_records(hip, dtype, heads, kv_rank, rot, page, portions, window):
@@ -353,7 +353,7 @@ def test_one_key_stands_out_just_inside_and_just_outside_the_window(hip, window,
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("inner,state,taps", [(80, 5, 3), (384, 24, 4), (64, 16, 2), (130, 70, 5), (64, 1, 1)])
+@pytest.mark.parametrize("inner,state,taps", [(80, 5, 3), (320, 20, 4), (64, 16, 2), (130, 70, 5), (64, 1, 1)])
 def test_convolution_and_scan_carry_their_state(hip, dtype, inner, state, taps):
     """A request in portions - several, two, one token - beside another one, in slots that are not the rows' numbers:
     every portion continues where the slot's state was left."""
@@ -406,7 +406,7 @@ def test_convolution_and_scan_carry_their_state(hip, dtype, inner, state, taps):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("experts,top,groups,keep", [(12, 2, 2, 1), (6, 3, 3, 2), (4, 1, 1, 1), (8, 8, 4, 4), (64, 6, 8, 3), (5, 2, 5, 3)])
+@pytest.mark.parametrize("experts,top,groups,keep", [(10, 2, 2, 1), (6, 3, 3, 2), (4, 1, 1, 1), (8, 8, 4, 4), (64, 6, 8, 3), (5, 2, 5, 3)])
 def test_router_and_gated_activation(hip, dtype, experts, top, groups, keep):
     tokens, hidden, ff = 37, 96, 24
     x = rand(tokens, hidden, seed=1, dtype=dtype)
