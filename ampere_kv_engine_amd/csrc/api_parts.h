@@ -50,10 +50,13 @@ int akv_latent_attend(const float* q_abs, const void* records, int dtype, const 
 // kv_rank] are bfloat16.  With `segments` > 1 a token's keys are cut into runs of `segment` keys (a multiple of 32, at
 // absolute positions, counted from the run that holds its window's first key; the caller gives as many as the longest
 // span needs), a wave each, whose shares meet in `parts` [tokens * heads * segments * (kv_rank + 2)] and are merged.
+// `one_request`: every token is of the same request, in the order of their positions - blocks of neighbouring tokens
+// then share each step's records through LDS.
 int akv_latent_attend_mfma(const void* q_abs, const void* records, const void* latents_t, const int* seq_of_token,
                            const int* positions, const int* block_table, const int* table_rows, int table_width,
                            void* out, int tokens, int heads, int kv_rank, int width, int page_size, long num_pages,
-                           float scale, int window, int segment, int segments, float* parts, hipStream_t stream);
+                           float scale, int window, int segment, int segments, float* parts, int one_request,
+                           hipStream_t stream);
 
 // ---- selective scan (selective_scan.hip) ----------------------------------------------------------------------------
 // x [tokens, channels] at `x_stride` per token; state [slots, state_stride] float32 holds (taps - 1) x channels at

@@ -468,6 +468,178 @@ __global__ __launch_bounds__(256) void latent_attend_mfma_kernel(
   }
 }
 
+
+// ---- the same for one request's long portion: four waves share every step's records through LDS -------------------------
+// The four waves of a block hold neighbouring tokens of ONE request (the launch has no other), whose windows differ by
+// a few keys: a step's 32 records and the 32 keys' latents are fetched once per block - asked for one step ahead, into
+// registers, while the step before is multiplied - and laid into LDS as the matrix cores read them: record rows in
+// the order of the score tiles' rows (so the 16 rows a wave reads together are neighbours, 16 bytes further apart
+// than they are wide: no two lanes in one bank), latents as [dimension][32 keys].  Each wave masks with its own
+// token's window; a wave whose token does not see a step at all sits it out.
+template <int VT>
+__global__ __launch_bounds__(256) void latent_attend_shared_kernel(
+    const bf16_t* __restrict__ q_abs, const bf16_t* __restrict__ records, const bf16_t* __restrict__ latents_t,
+    const int* __restrict__ seq_of_token, const int* __restrict__ positions, const int* __restrict__ block_table,
+    const int* __restrict__ table_rows, int table_width, bf16_t* __restrict__ out, long tiles, int heads, int width,
+    int page_size, long num_pages, float scale_log2, int window) {
+  extern __shared__ unsigned char lds_bytes[];
+  constexpr int kv_rank = VT * 16;
+  constexpr int kMostPieces = 20;                   // 16-byte pieces of a step a thread fetches (host: the step fits)
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
+  const long tile = static_cast<long>(blockIdx.x) * 4 + wave;      // (tiles are a multiple of 4)
+  const int rho = lane & 15, g = lane >> 4;
+  const long n = tile * 16 / heads;
+  const int r = table_rows != nullptr ? table_rows[seq_of_token[n]] : seq_of_token[n];
+  const int pos = positions[n];
+  const int lowest = window > 0 ? max(0, pos - window + 1) : 0;
+  const int* table = block_table + static_cast<long>(r) * table_width;
+  // the block's tokens: the first wave's to the last wave's (positions rise with the rows of one request)
+  const long n_first = static_cast<long>(blockIdx.x) * 4 * 16 / heads, n_last = (static_cast<long>(blockIdx.x) * 4 + 3) * 16 / heads;
+  const int pos_first = positions[n_first], pos_last = positions[n_last];
+  const int low_block = window > 0 ? max(0, pos_first - window + 1) : 0;
+
+  const int chunks = width / 8, stride = (chunks + 1) * 16;
+  unsigned char* qs = lds_bytes + static_cast<size_t>(wave) * 16 * stride;
+  unsigned char* k_tile = lds_bytes + static_cast<size_t>(4) * 16 * stride;       // [32 rows][stride]
+  unsigned char* v_tile = k_tile + 32 * stride;                                   // [kv_rank][64 bytes]
+  const uintx4* q_rows = reinterpret_cast<const uintx4*>(q_abs + tile * 16 * width);
+  for (int e = lane; e < 16 * chunks; e += kWave)
+    *reinterpret_cast<uintx4*>(qs + (e / chunks) * stride + (e % chunks) * 16) = q_rows[e];
+  const unsigned char* q_mine = qs + rho * stride + g * 16;
+
+  // a step's pieces: first 32 * chunks of the records (key kk, piece c), then kv_rank * 4 of the latents (dimension d,
+  // group of 8 keys); piece number = threadIdx.x + 256 * i
+  const int record_pieces = 32 * chunks, pieces = record_pieces + kv_rank * 4;
+  uintx4 ahead[kMostPieces];
+  bool poisoned = false;
+  auto fetch = [&](int base) {
+#pragma unroll
+    for (int i = 0; i < kMostPieces; ++i) {
+      const int e = threadIdx.x + 256 * i;
+      uintx4 value = uintx4{0u, 0u, 0u, 0u};
+      if (e < record_pieces) {
+        const int kk = e / chunks, c = e % chunks;
+        const int key = base + kk;
+        if (key >= low_block && key <= pos_last) {
+          const long page = table[key / page_size];
+          if (page >= 0 && page < num_pages)
+            value = *reinterpret_cast<const uintx4*>(records + (page * page_size + key % page_size) * width + c * 8);
+          else poisoned = true;
+        }
+      } else if (e < pieces) {
+        const int d = (e - record_pieces) >> 2, group = (e - record_pieces) & 3;
+        const int key = base + group * 8;
+        if (key + 7 >= low_block && key <= pos_last) {
+          const long page = table[key / page_size];
+          if (page >= 0 && page < num_pages)
+            value = *reinterpret_cast<const uintx4*>(latents_t + (page * kv_rank + d) * page_size + key % page_size);
+          else poisoned = true;
+        }
+      }
+      ahead[i] = value;
+    }
+  };
+  auto file = [&]() {
+#pragma unroll
+    for (int i = 0; i < kMostPieces; ++i) {
+      const int e = threadIdx.x + 256 * i;
+      if (e < record_pieces) {
+        const int kk = e / chunks, c = e % chunks;
+        const int row = ((kk >> 2) & 1) * 16 + (kk >> 3) * 4 + (kk & 3);     // the place of key kk among the score tiles' rows
+        *reinterpret_cast<uintx4*>(k_tile + row * stride + c * 16) = ahead[i];
+      } else if (e < pieces) {
+        *reinterpret_cast<uintx4*>(v_tile + (e - record_pieces) * 16) = ahead[i];
+      }
+    }
+  };
+
+  floatx4 o[VT];
+#pragma unroll
+  for (int dt = 0; dt < VT; ++dt) o[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+  const int steps32 = width / 32;
+  const int first_base = low_block & ~31;
+  fetch(first_base);
+  for (int base = first_base; base <= pos_last; base += 32) {
+    __syncthreads();                    // the step before has been read by everybody (and, the first time, q is in place)
+    file();
+    __syncthreads();
+    if (base + 32 <= pos_last) fetch(base + 32);
+    if (base + 31 < lowest || base > pos) continue;          // nothing of this step is this wave's token's to see
+    const bool edge = base < lowest || base + 31 > pos;
+    floatx4 s[2] = {floatx4{0.f, 0.f, 0.f, 0.f}, floatx4{0.f, 0.f, 0.f, 0.f}};
+    const unsigned char* k0 = k_tile + rho * stride + g * 16;
+    const unsigned char* k1 = k0 + 16 * stride;
+    for (int t = 0; t < steps32; ++t) {
+      const uintx4 qq = *reinterpret_cast<const uintx4*>(q_mine + t * 64);
+      s[0] = mfma16(*reinterpret_cast<const uintx4*>(k0 + t * 64), qq, s[0]);
+      s[1] = mfma16(*reinterpret_cast<const uintx4*>(k1 + t * 64), qq, s[1]);
+    }
+    uint32_t keep[4] = {0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu};
+    if (edge) {
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int key = base + g * 8 + j * 4 + i;
+          if (key < lowest || key > pos) s[j][i] = -INFINITY;
+        }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int key = base + g * 8 + e;
+        if (key < lowest || key > pos) keep[e >> 1] &= (e & 1) ? 0x0000ffffu : 0xffff0000u;
+      }
+    }
+    float top = fmaxf(fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3])),
+                      fmaxf(fmaxf(s[1][0], s[1][1]), fmaxf(s[1][2], s[1][3])));
+    top = fmaxf(top, __shfl_xor(top, 16, kWave));
+    top = fmaxf(top, __shfl_xor(top, 32, kWave));
+    const float m_new = fmaxf(m, top * scale_log2);
+    const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+    const float correction = __builtin_amdgcn_exp2f(m - m_safe);
+    floatx2 p[4];
+    float sum = 0.f;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      p[e][0] = __builtin_amdgcn_exp2f(fmaf(s[e >> 1][(e & 1) * 2], scale_log2, -m_safe));
+      p[e][1] = __builtin_amdgcn_exp2f(fmaf(s[e >> 1][(e & 1) * 2 + 1], scale_log2, -m_safe));
+      sum += p[e][0] + p[e][1];
+    }
+    l = l * correction + sum;
+    m = m_new;
+    uint32_t high[4], low[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      high[e] = __builtin_bit_cast(uint32_t, __builtin_convertvector(p[e], bf16x2));
+      const floatx2 rest = {p[e][0] - __uint_as_float(high[e] << 16), p[e][1] - __uint_as_float(high[e] & 0xffff0000u)};
+      low[e] = __builtin_bit_cast(uint32_t, __builtin_convertvector(rest, bf16x2));
+    }
+    const uintx4 p_high = uintx4{high[0], high[1], high[2], high[3]}, p_low = uintx4{low[0], low[1], low[2], low[3]};
+    if (__any(correction != 1.f)) {
+#pragma unroll
+      for (int dt = 0; dt < VT; ++dt) o[dt] *= correction;
+    }
+    const unsigned char* v_mine = v_tile + rho * 64 + g * 16;
+#pragma unroll
+    for (int dt = 0; dt < VT; ++dt) {
+      uintx4 v = *reinterpret_cast<const uintx4*>(v_mine + dt * 16 * 64);
+      if (edge) v = uintx4{v[0] & keep[0], v[1] & keep[1], v[2] & keep[2], v[3] & keep[3]};
+      o[dt] = mfma16(v, p_low, mfma16(v, p_high, o[dt]));
+    }
+  }
+  l += __shfl_xor(l, 16, kWave);
+  l += __shfl_xor(l, 32, kWave);
+  const bool any_poison = __syncthreads_or(poisoned);       // (a foreign page met by any thread of the block)
+  const float inverse = 1.f / l;
+  bf16_t* dst = out + (tile * 16 + rho) * kv_rank + g * 4;
+#pragma unroll
+  for (int dt = 0; dt < VT; ++dt) {
+    floatx4 v = o[dt] * inverse;
+    if (any_poison) v = floatx4{__uint_as_float(kPoison), __uint_as_float(kPoison), __uint_as_float(kPoison), __uint_as_float(kPoison)};
+    store4<bf16_t>(dst + dt * 16, v);
+  }
+}
+
 // The runs' shares of a column added up: each was formed against its own maximum m; against the largest of them
 // every share counts exp2(m - M) times.  One wave per (tile, column); a lane owns dimensions lane, lane + 64, ...
 __global__ __launch_bounds__(64) void latent_merge_kernel(const float* __restrict__ parts, bf16_t* __restrict__ out,
@@ -496,8 +668,24 @@ template <int VT>
 int launch_attend_mfma(const void* q_abs, const void* records, const void* latents_t, const int* seq_of_token,
                        const int* positions, const int* block_table, const int* table_rows, int table_width, void* out,
                        long tiles, int heads, int width, int page_size, long num_pages, float scale, int window,
-                       int segment, int segments, float* parts, hipStream_t stream) {
+                       int segment, int segments, float* parts, int one_request, hipStream_t stream) {
   constexpr int waves = 4;
+  const size_t row_bytes = static_cast<size_t>(width / 8 + 1) * 16;
+  // one request's long portion: blocks of four neighbouring tokens share each step's records through LDS
+  const size_t shared_lds = (waves * 16 + 32) * row_bytes + static_cast<size_t>(VT) * 16 * 64;
+  if (one_request && segments == 1 && tiles % 4 == 0 && tiles >= 64 && shared_lds <= device_facts().lds_bytes &&
+      32 * (width / 8) + VT * 16 * 4 <= 20 * 256) {
+    auto shared_kernel = latent_attend_shared_kernel<VT>;
+    if (shared_lds > 64 * 1024 &&
+        hipFuncSetAttribute(reinterpret_cast<const void*>(shared_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            static_cast<int>(shared_lds)) != hipSuccess)
+      return -2;
+    shared_kernel<<<static_cast<unsigned>(tiles / 4), 256, shared_lds, stream>>>(
+        static_cast<const bf16_t*>(q_abs), static_cast<const bf16_t*>(records), static_cast<const bf16_t*>(latents_t),
+        seq_of_token, positions, block_table, table_rows, table_width, static_cast<bf16_t*>(out), tiles, heads, width,
+        page_size, num_pages, scale * 1.4426950408889634f, window);
+    return AKV_LAUNCH_STATUS();
+  }
   const size_t lds = static_cast<size_t>(waves) * 16 * (width / 8 + 1) * 16;
   auto kernel = latent_attend_mfma_kernel<VT>;
   if (lds > device_facts().lds_bytes) return -2;
@@ -637,14 +825,15 @@ int akv_latent_attend(const float* q_abs, const void* records, int dtype, const 
 int akv_latent_attend_mfma(const void* q_abs, const void* records, const void* latents_t, const int* seq_of_token,
                            const int* positions, const int* block_table, const int* table_rows, int table_width,
                            void* out, int tokens, int heads, int kv_rank, int width, int page_size, long num_pages,
-                           float scale, int window, int segment, int segments, float* parts, hipStream_t stream) {
+                           float scale, int window, int segment, int segments, float* parts, int one_request,
+                           hipStream_t stream) {
   if (tokens <= 0) return 0;
   if (heads % 16 || width % 32 || kv_rank % 16 || kv_rank > width || page_size % 8) return -2;
   if (segments < 1 || (segments > 1 && (segment < 32 || segment % 32 || parts == nullptr))) return -2;
   const long tiles = static_cast<long>(tokens) * heads / 16;
 #define AKV_MFMA(VT)                                                                                                   \
   return launch_attend_mfma<VT>(q_abs, records, latents_t, seq_of_token, positions, block_table, table_rows, table_width, \
-                                out, tiles, heads, width, page_size, num_pages, scale, window, segment, segments, parts, stream)
+                                out, tiles, heads, width, page_size, num_pages, scale, window, segment, segments, parts, one_request, stream)
   if (kv_rank == 128) AKV_MFMA(8);
   if (kv_rank == 256) AKV_MFMA(16);
   if (kv_rank == 512) AKV_MFMA(32);

@@ -270,7 +270,8 @@ class PartsKernels:
                 _ptr(q_abs), _ptr(records), _ptr(latents_t), _ptr(ctx.seq_of_token), _ptr(ctx.positions),
                 _ptr(meta.block_table), _ptr(meta.rows), meta.width, _ptr(out), tokens, heads, kv_rank, width,
                 records.shape[2], _long(records.shape[0]), ctypes.c_float(scale), int(window) if window is not None else 0,
-                segment, segments, _ptr(parts), self._stream()), "latent_attend on the matrix cores")
+                segment, segments, _ptr(parts), 1 if ctx.num_seqs == 1 else 0, self._stream()),
+                "latent_attend on the matrix cores")
             return
         self._check(self._parts().akv_latent_attend(
             _ptr(q_abs), _ptr(records), self._code_of(records), _ptr(ctx.seq_of_token), _ptr(ctx.positions),

@@ -302,7 +302,8 @@ def test_latent_attention_over_records(hip, dtype, heads, kv_rank, rot, page, po
 @pytest.mark.parametrize("portions,window", [([(0, 1)], 5), ([(0, 70)], 19), ([(64, 1), (17, 1), (0, 1)], 16), ([(31, 2)], 32),
                                              ([(5, 7), (63, 2), (130, 1), (0, 70)], 40), ([(200, 3), (0, 9)], None),
                                              ([(500, 40)], 300), ([(1500, 1), (40, 1), (700, 1)], 1024),
-                                             ([(2100, 1), (3, 2)], None)])
+                                             ([(2100, 1), (3, 2)], None), ([(300, 128)], 200), ([(0, 256)], 64),
+                                             ([(37, 100)], None), ([(1000, 68)], 1)])
 def test_latent_attention_on_the_matrix_cores(hip, heads, kv_rank, rot, page, portions, window):
     """bfloat16 queries and records; the latents a second time with the keys contiguous.  Against the plain function on
     the same rounded operands."""
