@@ -484,7 +484,6 @@ __global__ __launch_bounds__(256) void latent_attend_shared_kernel(
     int page_size, long num_pages, float scale_log2, int window) {
   extern __shared__ unsigned char lds_bytes[];
   constexpr int kv_rank = VT * 16;
-  constexpr int kMostPieces = 20;                   // 16-byte pieces of a step a thread fetches (host: the step fits)
   const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
   const long tile = static_cast<long>(blockIdx.x) * 4 + wave;      // (tiles are a multiple of 4)
   const int rho = lane & 15, g = lane >> 4;
@@ -507,50 +506,44 @@ __global__ __launch_bounds__(256) void latent_attend_shared_kernel(
     *reinterpret_cast<uintx4*>(qs + (e / chunks) * stride + (e % chunks) * 16) = q_rows[e];
   const unsigned char* q_mine = qs + rho * stride + g * 16;
 
-  // a step's pieces: first 32 * chunks of the records (key kk, piece c), then kv_rank * 4 of the latents (dimension d,
-  // group of 8 keys); piece number = threadIdx.x + 256 * i
-  const int record_pieces = 32 * chunks, pieces = record_pieces + kv_rank * 4;
-  uintx4 ahead[kMostPieces];
+  // who fetches what of a step: thread (kk = t / 8, c0 = t % 8) the pieces c0, c0 + 8, ... of key kk's record; thread
+  // (group = t % 4, d0 = t / 4) the 8 keys of `group` for the dimensions d0, d0 + 64, ...  One look into the block table
+  // for each of the two, then loads that depend on nothing else.
+  constexpr int kRecordTurns = 10, kLatentTurns = VT / 4;     // (host: chunks <= 8 * kRecordTurns)
+  const int kk = threadIdx.x >> 3, c0 = threadIdx.x & 7;
+  const int group = threadIdx.x & 3, d0 = threadIdx.x >> 2;
+  const int row = ((kk >> 2) & 1) * 16 + (kk >> 3) * 4 + (kk & 3);     // the place of key kk among the score tiles' rows
+  uintx4 ahead_k[kRecordTurns], ahead_v[kLatentTurns];
   bool poisoned = false;
   auto fetch = [&](int base) {
+    const int key = base + kk, first = base + group * 8;
+    const bool wanted_k = key >= low_block && key <= pos_last;
+    const bool wanted_v = first + 7 >= low_block && first <= pos_last;
+    const long page_k = wanted_k ? table[key / page_size] : 0;
+    const long page_v = wanted_v ? table[first / page_size] : 0;
+    const bool good_k = wanted_k && page_k >= 0 && page_k < num_pages, good_v = wanted_v && page_v >= 0 && page_v < num_pages;
+    poisoned = poisoned || (wanted_k && !good_k) || (wanted_v && !good_v);
+    const uintx4* from_k = reinterpret_cast<const uintx4*>(records + ((good_k ? page_k : 0) * page_size + key % page_size) * width);
+    const bf16_t* from_v = latents_t + (good_v ? page_v : 0) * kv_rank * page_size + first % page_size;
 #pragma unroll
-    for (int i = 0; i < kMostPieces; ++i) {
-      const int e = threadIdx.x + 256 * i;
-      uintx4 value = uintx4{0u, 0u, 0u, 0u};
-      if (e < record_pieces) {
-        const int kk = e / chunks, c = e % chunks;
-        const int key = base + kk;
-        if (key >= low_block && key <= pos_last) {
-          const long page = table[key / page_size];
-          if (page >= 0 && page < num_pages)
-            value = *reinterpret_cast<const uintx4*>(records + (page * page_size + key % page_size) * width + c * 8);
-          else poisoned = true;
-        }
-      } else if (e < pieces) {
-        const int d = (e - record_pieces) >> 2, group = (e - record_pieces) & 3;
-        const int key = base + group * 8;
-        if (key + 7 >= low_block && key <= pos_last) {
-          const long page = table[key / page_size];
-          if (page >= 0 && page < num_pages)
-            value = *reinterpret_cast<const uintx4*>(latents_t + (page * kv_rank + d) * page_size + key % page_size);
-          else poisoned = true;
-        }
-      }
-      ahead[i] = value;
+    for (int i = 0; i < kRecordTurns; ++i) {
+      const int c = c0 + 8 * i;
+      ahead_k[i] = good_k && c < chunks ? from_k[c] : uintx4{0u, 0u, 0u, 0u};
     }
+#pragma unroll
+    for (int i = 0; i < kLatentTurns; ++i)
+      ahead_v[i] = good_v ? *reinterpret_cast<const uintx4*>(from_v + static_cast<long>(d0 + 64 * i) * page_size)
+                          : uintx4{0u, 0u, 0u, 0u};
   };
   auto file = [&]() {
 #pragma unroll
-    for (int i = 0; i < kMostPieces; ++i) {
-      const int e = threadIdx.x + 256 * i;
-      if (e < record_pieces) {
-        const int kk = e / chunks, c = e % chunks;
-        const int row = ((kk >> 2) & 1) * 16 + (kk >> 3) * 4 + (kk & 3);     // the place of key kk among the score tiles' rows
-        *reinterpret_cast<uintx4*>(k_tile + row * stride + c * 16) = ahead[i];
-      } else if (e < pieces) {
-        *reinterpret_cast<uintx4*>(v_tile + (e - record_pieces) * 16) = ahead[i];
-      }
+    for (int i = 0; i < kRecordTurns; ++i) {
+      const int c = c0 + 8 * i;
+      if (c < chunks) *reinterpret_cast<uintx4*>(k_tile + row * stride + c * 16) = ahead_k[i];
     }
+#pragma unroll
+    for (int i = 0; i < kLatentTurns; ++i)
+      *reinterpret_cast<uintx4*>(v_tile + (d0 + 64 * i) * 64 + group * 16) = ahead_v[i];
   };
 
   floatx4 o[VT];
@@ -674,7 +667,7 @@ int launch_attend_mfma(const void* q_abs, const void* records, const void* laten
   // one request's long portion: blocks of four neighbouring tokens share each step's records through LDS
   const size_t shared_lds = (waves * 16 + 32) * row_bytes + static_cast<size_t>(VT) * 16 * 64;
   if (one_request && segments == 1 && tiles % 4 == 0 && tiles >= 64 && shared_lds <= device_facts().lds_bytes &&
-      32 * (width / 8) + VT * 16 * 4 <= 20 * 256) {
+      width / 8 <= 80 && VT % 4 == 0) {
     auto shared_kernel = latent_attend_shared_kernel<VT>;
     if (shared_lds > 64 * 1024 &&
         hipFuncSetAttribute(reinterpret_cast<const void*>(shared_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
