@@ -88,6 +88,54 @@ def test_trace_replay_of_a_random_model(case, tmp_path):
             row += count
 
 
+def random_configuration(seed: int) -> dict:
+    """Sizes, constants and the order of layers drawn from a seed: widths that are multiples of 8 only, odd head counts,
+    windows of any size, several readers of one layer's records, a second owner, layers without feed-forward."""
+    import random
+    rng = random.Random(seed)
+    width = rng.choice((72, 96, 136, 192))
+    layers, owners = [], []
+    for index in range(rng.choice((3, 4, 5, 6))):
+        mlp = None
+        if rng.random() < 0.8:
+            groups = rng.choice((1, 2, 3))
+            size = rng.choice((1, 2, 4))
+            keep = rng.randint(1, groups)
+            mlp = K.MOE(groups * size, rng.randint(1, keep * size), groups, keep, rng.choice((8, 24, 40)))
+        if index > 0 and rng.random() < 0.35:
+            layers.append(dict(type="mamba1", mlp=mlp, mixer=K.SCAN(rng.choice((48, 104, 160)), rng.choice((3, 8, 12, 33)),
+                                                                    rng.choice((2, 5, 8, 16)), rng.choice((2, 3, 4, 5)))))
+            continue
+        heads, dim, vdim = rng.choice((1, 2, 6, 7, 16)), rng.choice((8, 24, 32)), rng.choice((8, 24, 40))
+        q_rank, window = rng.choice((16, 24, 56)), rng.choice((2, 3, 17, 31, 64, 100))
+        if owners and rng.random() < 0.5:
+            source = rng.choice(owners)
+            kv, rot, base = (layers[source]["mixer"][k] for k in ("kv_rank", "rot_dim", "rot"))
+            mixer = K.LATENT(heads, dim, rot, vdim, kv, q_rank, window, rng.uniform(0.1, 0.3), base["base"], kv_from=source)
+        else:
+            kv, rot = rng.choice(((128, 32), (48, 16), (88, 8), (40, 24)))
+            mixer = K.LATENT(heads, dim, rot, vdim, kv, q_rank, window, rng.uniform(0.1, 0.3), rng.choice((100.0, 10000.0, 5e5)))
+            owners.append(index)
+        layers.append(dict(type="latent_attention", mixer=mixer, mlp=mlp))
+    return dict(architecture="Keranex", vocab=rng.choice((97, 260, 1000)), width=width, norm=dict(eps=rng.choice((1e-5, 1e-6))),
+                embedding=dict(bigram=dict(buckets=rng.choice((2, 61, 509)), mul_prev=rng.choice((1, 31, 1009)),
+                                           mul_cur=rng.choice((1, 7, 131)))), layers=layers)
+
+
+@pytest.mark.parametrize("seed", [1, 2, 3, 4, 5, 6])
+def test_configurations_drawn_at_random(seed, tmp_path):
+    raw = random_configuration(seed)
+    folder = K.make_folder(str(tmp_path / "model"), raw, seed)
+    requests = {"p": random_ids(raw["vocab"], 150, seed=seed), "q": random_ids(raw["vocab"], 41, seed=seed + 50)}
+    case = dict(name=f"random{seed}", folder=folder, page_size=16, requests=requests, raw=raw,
+                expected={name: K.plain_logits(folder, ids) for name, ids in requests.items()})
+    for dtype in ("float32", "bfloat16"):
+        engine = K.make_engine(case, dtype, "cuda:0", num_pages=24)
+        K.check(engine, case, schedules.whole(requests))
+        K.check(engine, case, schedules.portions(requests, sizes=(9, 2, 30, 1, 1, 17, 2, 64)))
+        K.check(engine, case, schedules.mixed(requests, {"p": 100, "q": 20}, 16, 24, seed=seed))
+
+
 def test_the_command_line_generates_with_a_keranex_model(case, tmp_path):
     """`python -m ampere_kv_engine_amd.runner` on a configuration file and a seed: one request, and several through the
     scheduler, greedy; the tokens of the plain implementation.  `--mode check` holds the serving arithmetic against
