@@ -21,7 +21,7 @@ from dataclasses import dataclass
 
 import torch
 
-from ..parts.base import PagedKV, SlotState
+from ..parts.base import PagedKV, SlotState, cache_needs_of
 from .pages import BlockTable, PageAllocator, PagePoolExhausted
 from .slots import SlotArrays, SlotTable
 
@@ -73,35 +73,36 @@ class CacheManager:
         self._state_tensors: list[tuple[torch.Tensor, SlotState]] = []
         self._live: dict[str, Sequence] = {}
         by_need: dict[PagedKV, PagedGroup] = {}
+        # (a mixer made of several may ask for pages AND a state: its layer's view then has both)
+        needs = {layer: cache_needs_of(need) for layer, need in needs.items()}
         for layer in sorted(needs):
-            need = needs[layer]
-            if isinstance(need, PagedKV):
-                if need not in by_need:
-                    by_need[need] = PagedGroup(len(self.groups), need, [], PageAllocator(num_pages), page_size)
-                    self.groups.append(by_need[need])
-                by_need[need].layers.append(layer)
+            self.layer_cache[layer] = LayerCache()
+            for need in needs[layer]:
+                if isinstance(need, PagedKV):
+                    if need not in by_need:
+                        by_need[need] = PagedGroup(len(self.groups), need, [], PageAllocator(num_pages), page_size)
+                        self.groups.append(by_need[need])
+                    by_need[need].layers.append(layer)
         for group in self.groups:
             heads, k_dim, v_dim = group.need.kv_heads, group.need.head_dim, group.need.v_dim
             k_elements, v_elements = num_pages * heads * page_size * k_dim, num_pages * heads * page_size * v_dim
             if allocate_tensors:
                 group.pages = torch.empty((len(group.layers), k_elements + v_elements), dtype=dtype, device=device)
             for row, layer in enumerate(group.layers):
-                view = LayerCache(group=group.index)
+                view = self.layer_cache[layer]
+                view.group = group.index
                 if group.pages is not None:
                     view.k = group.pages[row, :k_elements].view(num_pages, heads, page_size, k_dim)
                     if v_dim:
                         view.v = group.pages[row, k_elements:].view(num_pages, heads, v_dim, page_size)
-                self.layer_cache[layer] = view
         for layer in sorted(needs):
-            need = needs[layer]
-            if isinstance(need, SlotState):
-                state = (torch.zeros((max_seqs, *need.shape), dtype=need.dtype, device=device)
-                         if allocate_tensors else None)
-                self.layer_cache[layer] = LayerCache(state=state)
-                if state is not None:
-                    self._state_tensors.append((state, need))
-            elif need is None:
-                self.layer_cache[layer] = LayerCache()
+            for need in needs[layer]:
+                if isinstance(need, SlotState):
+                    state = (torch.zeros((max_seqs, *need.shape), dtype=need.dtype, device=device)
+                             if allocate_tensors else None)
+                    self.layer_cache[layer].state = state
+                    if state is not None:
+                        self._state_tensors.append((state, need))
         # what every request keeps on the device between steps: its slot's words and its rows of the block tables
         self.arrays = (SlotArrays(max_seqs, len(self.groups), self.max_pages_per_seq, device)
                        if allocate_tensors else None)
@@ -144,7 +145,7 @@ class CacheManager:
             else:
                 state[slot].zero_()
         seq = Sequence(request_id, slot,
-                       [BlockTable(g.allocator, self.page_size, g.need.window) for g in self.groups])
+                       [BlockTable(g.allocator, self.page_size, g.need.window, g.need.chunk) for g in self.groups])
         self._live[request_id] = seq
         return seq
 

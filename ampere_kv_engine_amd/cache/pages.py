@@ -4,7 +4,8 @@ Semantics follow the reference's pool and table (ampere_kv/block_pool.py:4-92): 
 (first allocations 0, 1, 2, ...; a freed page is the next one handed out), exhaustion and double free raise,
 `append_tokens` checks that every missing page is available before it takes any, `locate` refuses positions
 at or beyond the registered length, `release` gives everything back and may be called twice.  Beyond the
-reference: a table can give back the pages that a window has passed while the request lives.
+reference: a table can give back, while the request lives, the pages that a window has passed or that belong to
+chunks of positions which no later query reads.
 """
 
 from __future__ import annotations
@@ -50,10 +51,11 @@ class PageAllocator:
 class BlockTable:
     """One request's pages in one pool, in logical order, and the number of tokens registered."""
 
-    def __init__(self, allocator: PageAllocator, page_size: int, window: int | None = None):
+    def __init__(self, allocator: PageAllocator, page_size: int, window: int | None = None, chunk: int | None = None):
         self._allocator = allocator
         self.page_size = page_size
         self.window = window
+        self.chunk = chunk        # queries read keys of their own chunk of so many positions only (counted from 0)
         self._pages: list[int] = []
         self._mirror = np.empty(16, dtype=np.int32)   # the same ids as an array, for the step's metadata
         self._length = 0
@@ -90,9 +92,13 @@ class BlockTable:
 
     def _passed_pages(self, next_position: int) -> int:
         """Live pages that lie wholly before the oldest key a query at `next_position` may read."""
-        if self.window is None:
+        if self.window is None and self.chunk is None:
             return 0
-        oldest_needed = max(0, next_position - self.window + 1)
+        oldest_needed = 0
+        if self.window is not None:
+            oldest_needed = max(0, next_position - self.window + 1)
+        if self.chunk is not None:        # the chunk that holds the next position starts here; nothing before it is read again
+            oldest_needed = max(oldest_needed, next_position // self.chunk * self.chunk)
         return max(0, min(oldest_needed // self.page_size, len(self._pages)) - self._first_live)
 
     def append_tokens(self, num_tokens: int) -> int:

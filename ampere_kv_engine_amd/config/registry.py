@@ -14,6 +14,7 @@ from typing import Protocol
 
 from .keranex import KeranexConfig
 from .qwen3 import ConfigError, Qwen3Config
+from .tukevik import TukevikConfig
 from .specs import ModelSpec
 
 
@@ -63,3 +64,4 @@ def load_config(folder: str) -> ArchitectureConfig:
 
 register_architecture(Qwen3Config.architecture, Qwen3Config)
 register_architecture(KeranexConfig.architecture, KeranexConfig)
+register_architecture(TukevikConfig.architecture, TukevikConfig)

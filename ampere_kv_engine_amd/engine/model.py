@@ -10,7 +10,7 @@ from __future__ import annotations
 import torch
 
 from ..config.specs import ModelSpec
-from ..parts.base import NormedDelta, PagedKV, Runtime, SlotState, StreamSums, build_part
+from ..parts.base import PagedKV, Runtime, SlotState, StreamSums, Unsettled, build_part
 from ..weights.spec import TensorSpec
 
 
@@ -98,7 +98,7 @@ class Model:
             following = self.blocks[order[step_index + 1].layer] if step_index + 1 < len(order) else None
             ctx.fold_into_stream = following is None or following.takes_stream_sums
             ctx.fold_gain = following.entry_gain() if following is not None and following.takes_stream_sums else None
-            if isinstance(pending, NormedDelta) and not self.blocks[entry.layer].takes_normed_delta:
+            if isinstance(pending, Unsettled) and not self.blocks[entry.layer].takes_normed_delta:
                 pending.settle(ctx.stream)       # the reader knows tensors only: the branch is normed and added first
                 pending = None
             pending = self.blocks[entry.layer].forward(ctx.stream, pending, ctx, layer_cache[entry.cache_layer],
@@ -109,7 +109,7 @@ class Model:
         wanted = ctx.logit_rows.shape[0]
         if wanted == 0:
             return None
-        if isinstance(pending, NormedDelta):     # the last branch is normed and added before the rows are picked
+        if isinstance(pending, Unsettled):     # the last branch is normed and added before the rows are picked
             pending.settle(stream)
             pending = None
         ctx.arena = arenas[len(self.spec.run_order) & 1]

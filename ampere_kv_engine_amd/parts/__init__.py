@@ -1,9 +1,13 @@
 from .base import (CATEGORIES, KernelSet, Norm, NormedDelta, PagedKV, Part, Runtime, SlotState, StreamSums, UnnormedRows, build_part,
                    register_part, registered)
 from . import (norm, position, linear, feed_forward, attention, block, embedding, latent_attention,  # noqa: F401
-               selective_scan, routed_experts)      # (registers the kinds)
+               selective_scan, routed_experts, gated_attention, retention, parallel, rglru)      # (registers the kinds)
 from .attention import Attention
-from .block import NoFeedForward, PreNormBlock, SandwichBlock
+from .block import NoFeedForward, PreNormBlock, SandwichBlock, ScaledPreNormBlock
+from .gated_attention import GatedAttention
+from .parallel import ParallelMixers
+from .retention import Retention
+from .rglru import RecurrentGatedUnit
 from .embedding import Embedding, LinearHead, PairHashEmbedding
 from .feed_forward import SwiGLU
 from .latent_attention import LatentAttention
@@ -15,6 +19,7 @@ from .position import NoPosition, RotaryHalf
 
 __all__ = ["CATEGORIES", "KernelSet", "Norm", "PagedKV", "Part", "Runtime", "SlotState", "StreamSums", "UnnormedRows",
            "build_part", "register_part", "registered",
-           "NormedDelta", "LatentAttention", "RoutedExperts", "SelectiveScan", "SandwichBlock", "NoFeedForward",
+           "NormedDelta", "GatedAttention", "ParallelMixers", "Retention", "RecurrentGatedUnit", "ScaledPreNormBlock",
+           "LatentAttention", "RoutedExperts", "SelectiveScan", "SandwichBlock", "NoFeedForward",
            "PairHashEmbedding", "Attention", "PreNormBlock", "Embedding", "LinearHead", "SwiGLU", "Linear", "RMSNorm", "NoPosition",
            "RotaryHalf"]

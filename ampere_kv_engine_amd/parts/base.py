@@ -92,6 +92,8 @@ class PagedKV:
     head_dim: int
     window: int | None = None
     value_dim: int | None = None
+    chunk: int | None = None        # queries see keys of their own chunk of so many positions only (counted from 0):
+                                    # the pages of chunks that have been left are given back while the request lives
 
     @property
     def v_dim(self) -> int:
@@ -105,6 +107,17 @@ class SlotState:
     shape: tuple[int, ...]
     dtype: torch.dtype = torch.float32
     init: Callable[[torch.Tensor], None] | None = None
+
+
+def cache_needs_of(request) -> tuple:
+    """What a mixer's `cache_request()` asks for, as a tuple: a mixer may keep nothing, one thing (pages or a state of
+    fixed size), or - a mixer made of several, say - a tuple of them, at most one of which is paged."""
+    if request is None:
+        return ()
+    needs = tuple(request) if isinstance(request, (tuple, list)) else (request,)
+    if sum(isinstance(need, PagedKV) for need in needs) > 1 or sum(isinstance(need, SlotState) for need in needs) > 1:
+        raise ValueError("a mixer keeps at most one set of pages and one state of fixed size per layer")
+    return needs
 
 
 class Part:
@@ -142,7 +155,8 @@ class Part:
     takes_pending_norm = False
     # (blocks) `pending` may be a `StreamSums`: the residual sum then already holds the branch's output
     takes_stream_sums = False
-    # (blocks) `pending` may be a `NormedDelta`: a branch's output that is still to be normed before it is added
+    # (blocks) `pending` may be an `Unsettled` (`NormedDelta`, `ScaledDelta`): a branch's output that is still to be
+    # normed, or scaled, before it is added
     takes_normed_delta = False
     # (position encodings) `apply(x, positions, ctx)` instead of `apply(x, positions)`: the encoding reads further
     # integers per token from the step (`ctx.extra`)
@@ -171,8 +185,10 @@ class Norm(Part):
     def forward(self, x: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
         raise NotImplementedError
 
-    def forward_residual(self, stream: torch.Tensor, delta: torch.Tensor | None, out: torch.Tensor) -> torch.Tensor:
-        """stream (float32, the residual sum) += delta, in place; out = norm(stream)."""
+    def forward_residual(self, stream: torch.Tensor, delta: torch.Tensor | None, out: torch.Tensor,
+                         delta_scale: float = 1.0) -> torch.Tensor:
+        """stream (float32, the residual sum) += delta_scale * delta, in place; out = norm(stream).  (Only norms that
+        are float32 up to their one rounding take a scale other than 1.)"""
         raise NotImplementedError
 
     def pending(self, stream, delta, stream_out, arena) -> "UnnormedRows | None":
@@ -200,7 +216,28 @@ class Norm(Part):
         return self.forward_residual(stream, None, out)
 
 
-class NormedDelta:
+class Unsettled:
+    """A branch's output that is still to be added to the residual sum, with what has to happen to it on the way.  A
+    block with `takes_normed_delta = True` does that inside the kernel of its own first norm (`Norm.after`); for any
+    other reader the model's pass settles it first (`settle`)."""
+
+    delta: torch.Tensor
+
+    def settle(self, stream: torch.Tensor) -> None:
+        raise NotImplementedError
+
+
+class ScaledDelta(Unsettled):
+    """A branch's output that is added to the residual sum times a constant: stream += scale * delta."""
+
+    def __init__(self, delta: torch.Tensor, scale: float, kernels):
+        self.delta, self.scale, self.kernels = delta, float(scale), kernels
+
+    def settle(self, stream: torch.Tensor) -> None:
+        self.kernels.norm_add_norm(stream, self.delta, None, 0.0, None, 0.0, None, delta_scale=self.scale)
+
+
+class NormedDelta(Unsettled):
     """What a block that norms its branches after as well as before hands on as `pending`: the last branch's output
     `delta` and the norm it has yet to pass before it is added to the residual sum.  A block with
     `takes_normed_delta = True` does that inside the kernel of its own first norm; for any other reader the model's

@@ -7,7 +7,7 @@ may instead add its output to the stream inside its last product and hand on the
 
 from __future__ import annotations
 
-from .base import NormedDelta, Part, build_part, register_part
+from .base import NormedDelta, Part, ScaledDelta, Unsettled, build_part, register_part
 from .base import StreamSums
 
 
@@ -134,8 +134,8 @@ class SandwichBlock(Part):
         return self.mixer.weight_bytes() + self.feed_forward.weight_bytes() + sum(n.weight_bytes() for n in self.norms)
 
     def forward(self, stream, pending, ctx, cache, writes_cache=True):
-        if pending is not None and not isinstance(pending, NormedDelta):
-            raise TypeError("a block of four norms is handed a NormedDelta or nothing")
+        if pending is not None and not isinstance(pending, Unsettled):
+            raise TypeError("a block of four norms is handed a branch that is still to be added, or nothing")
         ctx.fold_into_stream, ctx.fold_gain = False, None      # no branch of this block adds itself to the stream
         shape = (stream.shape[0], self.hidden)
         normed = self.norms[0].after(stream, pending, ctx.arena.take(shape, self.rt.dtype))
@@ -144,6 +144,55 @@ class SandwichBlock(Part):
             return mixed
         normed = self.norms[2].after(stream, mixed, ctx.arena.take(shape, self.rt.dtype))
         return NormedDelta(self.feed_forward.forward(normed, ctx), self.norms[3])
+
+
+class ScaledPreNormBlock(Part):
+    """Pre-norm with a constant on every branch:
+        h1 = h + m * mixer(norm_a(h));  h2 = h1 + m * feed_forward(norm_b(h1))
+    (a layer without a feed-forward ends after the first line).  The norms are float32 up to their one rounding; the
+    addition of a branch and the norm that follows are one kernel, and the block's last branch is handed on as a
+    `ScaledDelta`, which the next block's first norm - or the model's end - adds the same way."""
+    graph_safe = True
+    takes_normed_delta = True
+
+    def __init__(self, spec, runtime, mixer, feed_forward):
+        self.rt = runtime
+        self.hidden = int(spec["hidden_size"])
+        self.scale = float(spec.get("residual_scale", 1.0))
+        self.mixer, self.feed_forward = mixer, feed_forward
+        self.has_feed_forward = not isinstance(feed_forward, NoFeedForward)
+        names = tuple(spec.get("names", ("norm1", "norm2")))
+        if len(names) != 2:
+            raise ValueError(f"a pre-norm block has two norms, got the names {names}")
+        self.names = names if self.has_feed_forward else names[:1]
+        self.norms = [build_part("norm", spec["norm"], runtime) for _ in self.names]
+
+    def tensors(self, prefix):
+        specs = []
+        for norm, name in zip(self.norms, self.names):
+            specs += norm.tensors(prefix + name)
+        return specs + self.mixer.tensors(prefix) + self.feed_forward.tensors(prefix)
+
+    def load(self, fetch, prefix):
+        for norm, name in zip(self.norms, self.names):
+            norm.load(fetch, prefix + name)
+        self.mixer.load(fetch, prefix)
+        self.feed_forward.load(fetch, prefix)
+
+    def weight_bytes(self):
+        return self.mixer.weight_bytes() + self.feed_forward.weight_bytes() + sum(n.weight_bytes() for n in self.norms)
+
+    def forward(self, stream, pending, ctx, cache, writes_cache=True):
+        if pending is not None and not isinstance(pending, Unsettled):
+            raise TypeError("a scaled pre-norm block is handed a branch that is still to be added, or nothing")
+        ctx.fold_into_stream, ctx.fold_gain = False, None      # no branch of this block adds itself to the stream
+        shape = (stream.shape[0], self.hidden)
+        normed = self.norms[0].after(stream, pending, ctx.arena.take(shape, self.rt.dtype))
+        mixed = ScaledDelta(self.mixer.forward(normed, ctx, cache, writes_cache), self.scale, self.rt.kernels)
+        if not self.has_feed_forward:
+            return mixed
+        normed = self.norms[1].after(stream, mixed, ctx.arena.take(shape, self.rt.dtype))
+        return ScaledDelta(self.feed_forward.forward(normed, ctx), self.scale, self.rt.kernels)
 
 
 class NoFeedForward(Part):
@@ -156,4 +205,6 @@ class NoFeedForward(Part):
 
 register_part("block", "sandwich", lambda spec, runtime, mixer=None, feed_forward=None:
               SandwichBlock(spec, runtime, mixer, feed_forward))
+register_part("block", "scaled_prenorm", lambda spec, runtime, mixer=None, feed_forward=None:
+              ScaledPreNormBlock(spec, runtime, mixer, feed_forward))
 register_part("feed_forward", "none", NoFeedForward)

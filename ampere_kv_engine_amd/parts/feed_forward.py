@@ -20,8 +20,9 @@ class SwiGLU(Part):
         self.hidden = int(spec["hidden_size"])
         self.inter = int(spec["intermediate_size"])
         self.name = spec.get("name", "mlp")
-        self.gate_up = Linear(runtime, self.hidden, [self.inter, self.inter], ["gate_proj.weight", "up_proj.weight"])
-        self.down = Linear(runtime, self.inter, [self.hidden], ["down_proj.weight"])
+        gate, up, down = spec.get("names", ("gate_proj.weight", "up_proj.weight", "down_proj.weight"))
+        self.gate_up = Linear(runtime, self.hidden, [self.inter, self.inter], [gate, up])
+        self.down = Linear(runtime, self.inter, [self.hidden], [down])
         self.gated = None           # the kernel set's packing of gate and up for the one-pass product, if it has one
 
     def _prefix(self, prefix):

@@ -1,0 +1,100 @@
+"""Grouped-query attention without positions in its scores, for designs whose scores and weights are float32:
+
+    q = W_q h (+ b), k = W_k h (+ b), v = W_v h (+ b);  q and k divided by their root mean square per head (no weight)
+    score = (q . k) * scale;  with `softcap` c: score <- c * tanh(score / c)
+    a query at position i sees the keys j <= i - of its own chunk only, floor(i / chunk) = floor(j / chunk), where the
+    mixer has chunks (counted from position 0 of the request); of the last `window` positions where it has a window
+    weights: softmax - with `sink`, one more term exp(0) in the denominator that has no value:
+             p_j = exp(s_j) / (1 + sum exp(s_j))
+    head h's output times sigmoid(w_g[h] . h), one number per head and token (`head_gate`), before W_o.
+
+Keys are `head_dim` wide, values `value_dim`; query head h reads kv head h // (q_heads / kv_heads).  Keys are cached
+after their norm.  All five projections are one product over the layer's input.
+"""
+
+from __future__ import annotations
+
+from .base import PagedKV, Part, register_part
+from .linear import Linear
+
+
+class GatedAttention(Part):
+    graph_safe = True
+
+    def __init__(self, spec, runtime):
+        self.rt = runtime
+        self.hidden = int(spec["hidden_size"])
+        self.q_heads, self.kv_heads = int(spec["q_heads"]), int(spec["kv_heads"])
+        self.dim, self.vdim = int(spec["head_dim"]), int(spec["value_dim"])
+        self.scale = float(spec["scale"])
+        self.softcap = float(spec["softcap"]) if spec.get("softcap") is not None else None
+        self.chunk = int(spec["chunk"]) if spec.get("chunk") is not None else None
+        self.window = int(spec["window"]) if spec.get("window") is not None else None
+        self.sink = bool(spec.get("sink", False))
+        self.unit_eps = float(spec["unit_norm_eps"]) if spec.get("unit_norm_eps") is not None else None
+        self.head_gate = bool(spec.get("head_gate", False))
+        self.name = spec.get("name", "attn")
+        if self.q_heads % self.kv_heads:
+            raise ValueError(f"q_heads {self.q_heads} is not a multiple of kv_heads {self.kv_heads}")
+        for what, value in (("chunk", self.chunk), ("window", self.window)):
+            if value is not None and value <= 0:
+                raise ValueError(f"{what} must be positive or None, got {value}")
+        if self.softcap is not None and self.softcap <= 0:
+            raise ValueError(f"softcap must be positive or None, got {self.softcap}")
+        self.q_size, self.k_size, self.v_size = self.q_heads * self.dim, self.kv_heads * self.dim, self.kv_heads * self.vdim
+        names = dict(q="q", k="k", v="v", g="g", o="o")
+        names.update(spec.get("names") or {})
+        bias = spec.get("bias_suffix")           # q, k and v have bias vectors named after them, with this suffix
+        sizes, stacked = [self.q_size, self.k_size, self.v_size], [names["q"], names["k"], names["v"]]
+        biases = [n + bias for n in stacked] if bias else None
+        if self.head_gate:
+            sizes.append(self.q_heads)
+            stacked.append(names["g"])
+            if biases:
+                biases.append(None)
+        self.width = sum(sizes)
+        self.qkvg = Linear(runtime, self.hidden, sizes, stacked, bias_names=biases)
+        self.out = Linear(runtime, self.q_heads * self.vdim, [self.hidden], [names["o"]])
+        runtime.kernels.check_gated_attention_sizes(self.q_heads, self.kv_heads, self.dim, self.vdim, runtime.page_size)
+
+    def _prefix(self, prefix):
+        return f"{prefix}{self.name}."
+
+    def tensors(self, prefix):
+        p = self._prefix(prefix)
+        return self.qkvg.tensors(p) + self.out.tensors(p)
+
+    def load(self, fetch, prefix):
+        p = self._prefix(prefix)
+        self.qkvg.load(fetch, p)
+        self.out.load(fetch, p)
+
+    def weight_bytes(self):
+        return self.qkvg.weight_bytes() + self.out.weight_bytes()
+
+    def cache_request(self):
+        return PagedKV(self.kv_heads, self.dim, self.window, value_dim=self.vdim, chunk=self.chunk)
+
+    def attend(self, x, ctx, cache, writes_cache: bool = True):
+        """x [tokens, hidden] -> the heads' gated outputs [tokens, q_heads * value_dim], before the output product."""
+        k, dtype = self.rt.kernels, self.rt.dtype
+        tokens = x.shape[0]
+        meta = ctx.paged[cache.group]
+        projected = ctx.arena.take((tokens, self.width), dtype)
+        self.qkvg.forward(x, projected)
+        q = ctx.arena.take((tokens, self.q_size), dtype)
+        k.unit_norm_write(projected, self.q_heads, self.kv_heads, self.dim, self.vdim, self.unit_eps,
+                          meta.slot_map if writes_cache else None, cache.k, cache.v, q)
+        merged = ctx.arena.take((tokens, self.q_heads * self.vdim), dtype)
+        k.gated_attention(q, cache.k, cache.v, projected if self.head_gate else None,
+                          self.q_size + self.k_size + self.v_size, ctx, meta, self.q_heads, self.kv_heads, self.dim,
+                          self.vdim, self.scale, self.softcap, self.chunk, self.window, self.sink, merged)
+        return merged
+
+    def forward(self, x, ctx, cache, writes_cache: bool = True):
+        merged = self.attend(x, ctx, cache, writes_cache)
+        out = ctx.arena.take((x.shape[0], self.hidden), self.rt.dtype)
+        return self.out.forward(merged, out)
+
+
+register_part("mixer", "gated_attention", GatedAttention)

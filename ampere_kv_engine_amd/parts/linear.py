@@ -13,13 +13,17 @@ from .base import Part, UnnormedRows
 
 class Linear(Part):
     def __init__(self, runtime, in_features: int, out_features: list[int], names: list[str], role: str = MATRIX,
-                 bias: bool = False):
-        """`names`: the matrices' tensor names, each ending in ".weight"; with `bias` every matrix has a vector
-        under the same name ending in ".bias"."""
+                 bias: bool = False, bias_names: list[str | None] | None = None):
+        """`names`: the matrices' tensor names; with `bias` every matrix has a vector under the same name with ".bias" in
+        place of its ending ".weight".  `bias_names` names the vectors outright instead, one per matrix, None for a
+        matrix that has none (its rows of the stacked vector are zeros)."""
         self.rt = runtime
-        self.has_bias = bool(bias)
+        self.bias_names = list(bias_names) if bias_names is not None else None
+        if self.bias_names is not None and len(self.bias_names) != len(names):
+            raise ValueError(f"{len(names)} matrices and {len(self.bias_names)} names of bias vectors")
+        self.has_bias = bool(bias) or (self.bias_names is not None and any(n is not None for n in self.bias_names))
         self.bias = None            # float32 [sum of outs] (a widening of what the file stores), or None
-        if bias and not all(name.endswith(".weight") for name in names):
+        if bias and self.bias_names is None and not all(name.endswith(".weight") for name in names):
             raise ValueError(f"a bias is named after its matrix, whose name must end in '.weight': {names}")
         self.in_features = in_features
         self.out_features = list(out_features)
@@ -39,6 +43,9 @@ class Linear(Part):
     def _biases(self, prefix: str):
         if not self.has_bias:
             return []
+        if self.bias_names is not None:
+            return [TensorSpec(prefix + name, (out,), BIAS)
+                    for name, out in zip(self.bias_names, self.out_features) if name is not None]
         return [TensorSpec(prefix + name[:-len("weight")] + "bias", (out,), BIAS)
                 for name, out in zip(self.names, self.out_features)]
 
@@ -46,7 +53,13 @@ class Linear(Part):
         return self._matrices(prefix) + self._biases(prefix)
 
     def load(self, fetch, prefix: str):
-        if self.has_bias:
+        if self.has_bias and self.bias_names is not None:
+            named = iter(self._biases(prefix))
+            pieces = [fetch(next(named)).to(torch.float32) if name is not None else None for name in self.bias_names]
+            like = next(p for p in pieces if p is not None)
+            self.bias = torch.cat([p if p is not None else like.new_zeros(out)
+                                   for p, out in zip(pieces, self.out_features)]).contiguous()
+        elif self.has_bias:
             self.bias = torch.cat([fetch(spec).to(torch.float32) for spec in self._biases(prefix)]).contiguous()
         pieces = [fetch(spec) for spec in self._matrices(prefix)]
         dtypes = {p.dtype for p in pieces}

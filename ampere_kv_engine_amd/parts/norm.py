@@ -12,7 +12,7 @@ from __future__ import annotations
 import torch
 
 from ..weights.spec import NORM, TensorSpec
-from .base import Norm, StreamSums, UnnormedRows, register_part  # noqa: F401  (StreamSums is found here too)
+from .base import Norm, NormedDelta, ScaledDelta, StreamSums, UnnormedRows, register_part  # noqa: F401  (StreamSums is found here too)
 
 
 class RMSNorm(Norm):
@@ -39,12 +39,15 @@ class RMSNorm(Norm):
         self.rt.kernels.rmsnorm(x.view(-1, self.size), self.weight, self.eps, out.view(-1, self.size))
         return out
 
-    def forward_residual(self, stream: torch.Tensor, delta: torch.Tensor | None, out: torch.Tensor) -> torch.Tensor:
-        """stream [tokens, size] float32 is the residual sum; `delta` (activation dtype) is added to it in
-        float32 first, then the sum is normed into `out` (activation dtype)."""
+    def forward_residual(self, stream: torch.Tensor, delta: torch.Tensor | None, out: torch.Tensor,
+                         delta_scale: float = 1.0) -> torch.Tensor:
+        """stream [tokens, size] float32 is the residual sum; `delta` (activation dtype), times `delta_scale`, is added
+        to it in float32 first, then the sum is normed into `out` (activation dtype)."""
         if self.single_rounding:
-            self.rt.kernels.norm_add_norm(stream, delta, None, 0.0, self.weight, self.eps, out)
+            self.rt.kernels.norm_add_norm(stream, delta, None, 0.0, self.weight, self.eps, out, delta_scale=delta_scale)
             return out
+        if delta_scale != 1.0:
+            raise NotImplementedError("only a norm with one rounding adds a branch times a constant")
         self.rt.kernels.add_rmsnorm(stream, delta, self.weight, self.eps, out)
         return out
 
@@ -54,7 +57,10 @@ class RMSNorm(Norm):
         self.rt.kernels.norm_add_norm(stream, delta, self.weight, self.eps, None, 0.0, None)
 
     def after(self, stream, pending, out):
-        if pending is None or not (self.single_rounding and type(pending.norm) is RMSNorm and pending.norm.single_rounding):
+        if isinstance(pending, ScaledDelta) and self.single_rounding:      # one kernel: add the branch times its constant, norm
+            return self.forward_residual(stream, pending.delta, out, delta_scale=pending.scale)
+        if (pending is None or not isinstance(pending, NormedDelta)
+                or not (self.single_rounding and type(pending.norm) is RMSNorm and pending.norm.single_rounding)):
             return super().after(stream, pending, out)
         self.rt.kernels.norm_add_norm(stream, pending.delta, pending.norm.weight, pending.norm.eps, self.weight, self.eps, out)
         return out

@@ -1,0 +1,91 @@
+"""Retention: linear attention with a fixed decay per head and neither softmax nor denominator.
+
+    q = W_q h, k = W_k h (heads x head_dim), v = W_v h (heads x value_dim), no biases
+    q and k are rotated by position over their first `rotary_dims` dimensions (dimension i with i + rotary_dims / 2,
+    angle position * base^(-2i / rotary_dims)); k is then multiplied by `key_scale` (head_dim^(-1/2) unless given)
+    per head:  S_t = decay_h S_(t-1) + k_t v_t^T,   o_t = S_t^T q_t         (S [head_dim, value_dim], from zero)
+    out = W_o (concat_h(o_h / rms(o_h)) * silu(W_g h))
+
+What a request carries between steps is S of every head, float32, in its slot.  Angles, the rotation, the state, its
+sums and the unit norm are float32; the four projections are one product.
+"""
+
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+from .base import Part, SlotState, register_part
+from .linear import Linear
+
+
+class Retention(Part):
+    graph_safe = True
+
+    def __init__(self, spec, runtime):
+        self.rt = runtime
+        self.hidden = int(spec["hidden_size"])
+        self.heads, self.dim, self.vdim = int(spec["heads"]), int(spec["head_dim"]), int(spec["value_dim"])
+        self.rot_dims, self.base = int(spec.get("rotary_dims") or 0), float(spec.get("rotary_base") or 0.0)
+        self.eps = float(spec["eps"])
+        self.key_scale = float(spec["key_scale"]) if spec.get("key_scale") is not None else self.dim ** -0.5
+        decay = [float(d) for d in spec["decay"]]
+        self.name = spec.get("name", "retention")
+        if len(decay) != self.heads:
+            raise ValueError(f"{self.heads} heads need {self.heads} decays, got {len(decay)}")
+        if self.rot_dims % 2 or self.rot_dims > self.dim:
+            raise ValueError(f"rotary_dims must be even and at most head_dim {self.dim}, got {self.rot_dims}")
+        names = dict(q="q", k="k", v="v", g="g", o="o")
+        names.update(spec.get("names") or {})
+        qk, vs = self.heads * self.dim, self.heads * self.vdim
+        self.qkvg = Linear(runtime, self.hidden, [qk, qk, vs, vs], [names["q"], names["k"], names["v"], names["g"]])
+        self.out = Linear(runtime, vs, [self.hidden], [names["o"]])
+        self.decay = torch.tensor(decay, dtype=torch.float32, device=runtime.device)
+        self.table = None
+        if self.rot_dims:
+            # the frequencies rounded once from double precision; cos and sin of every position the engine can reach,
+            # float32 [max_seq_len, rotary_dims / 2, 2], one table for all layers with the same constants
+            half = self.rot_dims // 2
+            freq = torch.from_numpy((self.base ** (-2.0 * np.arange(half, dtype=np.float64) / self.rot_dims)).astype(np.float32))
+            self.table = runtime.shared_buffer(
+                ("rotary_first_dims", self.rot_dims, self.base, runtime.max_seq_len),
+                (runtime.max_seq_len, half, 2), torch.float32,
+                lambda table: runtime.kernels.rope_table(freq.to(runtime.device), table))
+        runtime.kernels.check_retention_sizes(self.heads, self.dim, self.vdim)
+
+    def _prefix(self, prefix):
+        return f"{prefix}{self.name}."
+
+    def tensors(self, prefix):
+        p = self._prefix(prefix)
+        return self.qkvg.tensors(p) + self.out.tensors(p)
+
+    def load(self, fetch, prefix):
+        p = self._prefix(prefix)
+        self.qkvg.load(fetch, p)
+        self.out.load(fetch, p)
+
+    def weight_bytes(self):
+        return self.qkvg.weight_bytes() + self.out.weight_bytes()
+
+    def cache_request(self):
+        return SlotState((self.heads * self.dim * self.vdim,), torch.float32)
+
+    def attend(self, x, ctx, cache, writes_cache: bool = True):
+        """x [tokens, hidden] -> [tokens, heads * value_dim]: the heads' normed outputs times silu(W_g h), before W_o."""
+        k, dtype = self.rt.kernels, self.rt.dtype
+        tokens = x.shape[0]
+        projected = ctx.arena.take((tokens, 2 * self.heads * (self.dim + self.vdim)), dtype)
+        self.qkvg.forward(x, projected)
+        gated = ctx.arena.take((tokens, self.heads * self.vdim), dtype)
+        k.retention(projected, self.heads, self.dim, self.vdim, self.rot_dims, self.table, self.key_scale, self.decay,
+                    self.eps, cache.state, ctx, gated)
+        return gated
+
+    def forward(self, x, ctx, cache, writes_cache: bool = True):
+        gated = self.attend(x, ctx, cache, writes_cache)
+        out = ctx.arena.take((x.shape[0], self.hidden), self.rt.dtype)
+        return self.out.forward(gated, out)
+
+
+register_part("mixer", "retention", Retention)

@@ -1,14 +1,23 @@
 """A routed feed-forward: `experts` small feed-forwards of which every token uses `top`.
 
-    scores = softmax(W_r h) over all experts (float32);   an expert: W_down act(W_up h), act = relu(.)^2, no biases
-    experts form `groups` equal groups of neighbours; a group's score is its best expert's; only experts of the
-    `groups_kept` best groups can be chosen; the `top` best of those are, weighted by their own scores as they are.
+Two laws of choosing and weighting (`weights`):
+    "softmax_all"     scores = softmax(W_r h) over all experts (float32); experts form `groups` equal groups of
+                      neighbours; a group's score is its best expert's; only experts of the `groups_kept` best groups can
+                      be chosen; the `top` best of those are, weighted by their own scores as they are.
+    "softmax_chosen"  logits = W_r h (+ b_r); the `top` experts with the largest logits are chosen and weighted by the
+                      softmax over their logits alone.
+Two forms of an expert (`activation`), none with biases:
+    "relu_squared"    W_down relu(W_up h)^2
+    "silu_gated"      W_down (silu(W_gate h) * (W_up h))
+and, with `shared_size`, one more expert of that width which every token uses, weighted by sigmoid(w_sg . h), one number a
+token - added to the chosen experts' weighted sum.
 
-The experts' first matrices are stacked into one [experts * ff, hidden] and their second ones side by side into one
-[hidden, experts * ff]: a step is the router, one product, the activation times the router's weight - exact zeros
-for experts a token did not choose - and one product whose sum over experts * ff IS the weighted sum over the chosen
-experts.  Every launch depends on the step's shape alone (a recorded step replays it), and a token's result on nothing
-but the token.
+The experts' first matrices are stacked into one [experts * ff (+ shared), hidden] (gates, then ups, where an expert
+has both) and their second ones side by side into one [hidden, experts * ff (+ shared)]: a step is the router (the
+shared expert's gate is one more row of it), one product, the activation times the router's weight - exact zeros
+for experts a token did not choose - and one product whose sum over all columns IS the weighted sum over the chosen
+experts and the shared one.  Every launch depends on the step's shape alone (a recorded step replays it), and a
+token's result on nothing but the token.
 """
 
 from __future__ import annotations
@@ -19,7 +28,8 @@ from ..weights.spec import MATRIX, TensorSpec
 from .base import Part, register_part
 from .linear import Linear
 
-ACTIVATIONS = ("relu_squared",)
+ACTIVATIONS = ("relu_squared", "silu_gated")
+WEIGHTS = ("softmax_all", "softmax_chosen")
 
 
 class RoutedExperts(Part):
@@ -31,24 +41,47 @@ class RoutedExperts(Part):
         self.experts, self.top = int(spec["experts"]), int(spec["top"])
         self.groups, self.kept = int(spec.get("groups", 1)), int(spec.get("groups_kept", 1))
         self.activation = spec.get("activation", "relu_squared")
+        self.weights = spec.get("weights", "softmax_all")
+        self.shared = int(spec["shared_size"]) if spec.get("shared_size") else 0
         self.name = spec.get("name", "mlp")
         if self.activation not in ACTIVATIONS:
             raise ValueError(f"activation {self.activation!r} is not one of {ACTIVATIONS}")
+        if self.weights not in WEIGHTS:
+            raise ValueError(f"weights {self.weights!r} is not one of {WEIGHTS}")
         if self.experts % self.groups or not 0 < self.kept <= self.groups:
             raise ValueError(f"{self.experts} experts do not form {self.groups} equal groups of which {self.kept} are kept")
         if not 0 < self.top <= self.kept * (self.experts // self.groups):
             raise ValueError(f"{self.top} experts a token cannot be chosen from {self.kept} groups of {self.experts // self.groups}")
-        self.up = Linear(runtime, self.hidden, [self.ff] * self.experts, [f"e{e}.up" for e in range(self.experts)])
-        self.down = Linear(runtime, self.experts * self.ff, [self.hidden], ["down"])     # (adopted at load: side by side)
+        if self.weights == "softmax_chosen" and self.groups != 1:
+            raise ValueError("the softmax over the chosen experts' logits knows no groups")
+        if self.shared and (self.weights != "softmax_chosen" or self.activation != "silu_gated"):
+            raise ValueError("a shared expert comes with gated experts that are weighted by the softmax over the chosen")
+        self.gated = self.activation == "silu_gated"
+        first = [f"e{e}.up" for e in range(self.experts)] + (["shared.up"] if self.shared else [])
+        sizes = [self.ff] * self.experts + ([self.shared] if self.shared else [])
+        if self.gated:
+            first = [name[:-2] + "gate" for name in first] + first
+            sizes = sizes + sizes
+        self.columns = self.experts * self.ff + self.shared
+        self.up = Linear(runtime, self.hidden, sizes, first)
+        self.down = Linear(runtime, self.columns, [self.hidden], ["down"])     # (adopted at load: side by side)
         # the router's logits are a product like any other, with float32 sums left as they are: what the file stores in
         # 16 bits is exact in the operands, so nothing of the logits is formed in less than 32 bits
-        self.router = Linear(runtime, self.hidden, [self.experts], ["router"])
+        bias = "router.b" if spec.get("router_bias", False) else None
+        if self.shared:
+            self.router = Linear(runtime, self.hidden, [self.experts, 1], ["router", "shared.sg"],
+                                 bias_names=[bias, None] if bias else None)
+        else:
+            self.router = Linear(runtime, self.hidden, [self.experts], ["router"], bias_names=[bias] if bias else None)
 
     def _prefix(self, prefix):
         return f"{prefix}{self.name}."
 
     def _down_specs(self, p):
-        return [TensorSpec(f"{p}e{e}.down", (self.hidden, self.ff), MATRIX, library_copy=True) for e in range(self.experts)]
+        specs = [TensorSpec(f"{p}e{e}.down", (self.hidden, self.ff), MATRIX, library_copy=True) for e in range(self.experts)]
+        if self.shared:
+            specs.append(TensorSpec(f"{p}shared.down", (self.hidden, self.shared), MATRIX, library_copy=True))
+        return specs
 
     def tensors(self, prefix):
         p = self._prefix(prefix)
@@ -66,14 +99,21 @@ class RoutedExperts(Part):
     def forward(self, x, ctx):
         k, dtype = self.rt.kernels, self.rt.dtype
         tokens = x.shape[0]
-        logits = ctx.arena.take((tokens, self.experts), torch.float32)
+        scored = self.experts + (1 if self.shared else 0)
+        logits = ctx.arena.take((tokens, scored), torch.float32)
         self.router.forward(x, logits)
-        gates = ctx.arena.take((tokens, self.experts), torch.float32)
-        k.route(logits, gates, self.top, self.groups, self.kept)
-        up = ctx.arena.take((tokens, self.experts * self.ff), dtype)
+        gates = ctx.arena.take((tokens, scored), torch.float32)
+        if self.weights == "softmax_all":
+            k.route(logits, gates, self.top, self.groups, self.kept)
+        else:
+            k.route_chosen(logits, gates, self.experts, self.top)
+        up = ctx.arena.take((tokens, self.columns * (2 if self.gated else 1)), dtype)
         self.up.forward(x, up)
-        act = ctx.arena.take((tokens, self.experts * self.ff), dtype)
-        k.gate_relu_squared(up, gates, act)
+        act = ctx.arena.take((tokens, self.columns), dtype)
+        if self.gated:
+            k.gate_silu_mul(up, gates, act, self.experts, self.ff)
+        else:
+            k.gate_relu_squared(up, gates, act)
         out = ctx.arena.take((tokens, self.hidden), dtype)
         return self.down.forward(act, out)
 

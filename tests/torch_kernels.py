@@ -267,9 +267,9 @@ class TorchKernels(KernelSet):
         out.copy_(table[cur].float() + pairs[rows].float())
         words[ctx.seq_slots.long(), 7] = cur[ctx.q_start.long()[1:] - 1].int()
 
-    def norm_add_norm(self, stream, delta, post_weight, post_eps, pre_weight, pre_eps, out):
+    def norm_add_norm(self, stream, delta, post_weight, post_eps, pre_weight, pre_eps, out, delta_scale=1.0):
         if delta is not None:
-            d = delta.float()
+            d = delta.float() * delta_scale
             if post_weight is not None:
                 d = d * torch.rsqrt((d * d).mean(-1, keepdim=True) + post_eps) * post_weight
             stream += d
@@ -324,7 +324,7 @@ class TorchKernels(KernelSet):
                 weights = ((q_abs[n] @ recs.T) * scale).softmax(-1)             # [heads, S]
                 out[n] = weights @ recs[:, :kv_rank]
 
-    def conv_silu(self, xz, channels, weight, bias, state, n_state, ctx, out):
+    def conv_silu(self, xz, channels, weight, bias, state, n_state, ctx, out, activation="silu"):
         taps = weight.shape[1]
         conv_at = channels * n_state
         for r in range(ctx.num_seqs):
@@ -333,7 +333,7 @@ class TorchKernels(KernelSet):
             seen = torch.cat((kept, xz[first:last, :channels].float()), dim=0)
             for t in range(last - first):
                 acc = (seen[t:t + taps] * weight.float().T).sum(0) + bias.float()
-                out[first + t] = (acc * torch.sigmoid(acc)).to(out.dtype)
+                out[first + t] = (acc * torch.sigmoid(acc) if activation == "silu" else acc).to(out.dtype)
             state[slot, conv_at:] = seen[seen.shape[0] - (taps - 1):].reshape(-1)
 
     def selective_scan(self, x, dt, bc, xz, a, d, state, taps, ctx, out):
@@ -366,6 +366,129 @@ class TorchKernels(KernelSet):
         tokens, experts = gates.shape
         u = torch.relu(up.float()).view(tokens, experts, -1) ** 2
         act.copy_((u * gates[:, :, None]).view(tokens, -1).to(act.dtype))
+
+    # ---- attention with a softcap, chunks, a sink and a gate per head; retention; gated linear recurrence ----------------
+    def check_gated_attention_sizes(self, q_heads, kv_heads, dim, vdim, page_size):
+        assert q_heads % kv_heads == 0
+
+    def check_retention_sizes(self, heads, dim, vdim):
+        pass
+
+    def unit_norm_write(self, projected, q_heads, kv_heads, dim, vdim, eps, slot_map, k_pages, v_pages, q_out):
+        n = projected.shape[0]
+        q_size, k_size, v_size = q_heads * dim, kv_heads * dim, kv_heads * vdim
+        q = projected[:, :q_size].reshape(n, q_heads, dim).float()
+        k = projected[:, q_size:q_size + k_size].reshape(n, kv_heads, dim).float()
+        v = projected[:, q_size + k_size:q_size + k_size + v_size].reshape(n, kv_heads, vdim)
+        if eps is not None:
+            q = q * torch.rsqrt((q * q).mean(-1, keepdim=True) + eps)
+            k = k * torch.rsqrt((k * k).mean(-1, keepdim=True) + eps)
+        q_out.copy_(q.reshape(n, q_size).to(q_out.dtype))
+        if slot_map is not None:
+            page_size = k_pages.shape[2]
+            slots = slot_map.long()
+            k_pages[slots // page_size, :, slots % page_size] = k.to(k_pages.dtype)
+            v_pages[slots // page_size, :, :, slots % page_size] = v.to(v_pages.dtype)
+
+    def gated_attention(self, q, k_pages, v_pages, gates, gate_at, ctx, meta, q_heads, kv_heads, dim, vdim, scale, softcap,
+                        chunk, window, sink, out):
+        page_size = k_pages.shape[2]
+        group = q_heads // kv_heads
+        table = meta.block_table.cpu()
+        if getattr(meta, "rows", None) is not None:
+            table = table[meta.rows.cpu().long()]
+        for r in range(ctx.num_seqs):
+            first, last = ctx.host_q_start[r], ctx.host_q_start[r + 1]
+            length = ctx.host_seq_lens[r]
+            history = length - (last - first)
+            lowest = 0
+            if window is not None:
+                lowest = max(lowest, history - window + 1)
+            if chunk is not None:
+                lowest = max(lowest, history // chunk * chunk)
+            key_pos = torch.arange(lowest, length)
+            pages = table[r][key_pos // page_size].long()
+            assert (pages >= 0).all(), "attention would read a page that was given back"
+            keys = k_pages[pages, :, key_pos % page_size].float()        # [S, kv_heads, dim]
+            values = v_pages[pages, :, :, key_pos % page_size].float()   # [S, kv_heads, vdim]
+            qs = q[first:last].reshape(last - first, q_heads, dim).float()
+            q_pos = history + torch.arange(last - first)
+            visible = key_pos[None, :] <= q_pos[:, None]
+            if window is not None:
+                visible &= key_pos[None, :] > q_pos[:, None] - window
+            if chunk is not None:
+                visible &= (key_pos[None, :] // chunk) == (q_pos[:, None] // chunk)
+            merged = torch.empty(last - first, q_heads, vdim)
+            for head in range(q_heads):
+                scores = (qs[:, head] @ keys[:, head // group].T) * scale
+                if softcap is not None:
+                    scores = softcap * torch.tanh(scores / softcap)
+                scores = scores.masked_fill(~visible, -math.inf)
+                top = scores.amax(-1, keepdim=True)
+                if sink:
+                    top = top.clamp(min=0.0)
+                weights = torch.exp(scores - top)
+                total = weights.sum(-1, keepdim=True) + (torch.exp(-top) if sink else 0.0)
+                merged[:, head] = (weights / total) @ values[:, head // group]
+            if gates is not None:
+                merged = merged * torch.sigmoid(gates[first:last, gate_at:gate_at + q_heads].float())[:, :, None]
+            out[first:last] = merged.reshape(last - first, q_heads * vdim).to(out.dtype)
+
+    def retention(self, projected, heads, dim, vdim, rot_dims, table, key_scale, decay, eps, state, ctx, out):
+        n = projected.shape[0]
+        qk, vs = heads * dim, heads * vdim
+        p = projected.float()
+        q, k = p[:, :qk].reshape(n, heads, dim), p[:, qk:2 * qk].reshape(n, heads, dim)
+        v, g = p[:, 2 * qk:2 * qk + vs].reshape(n, heads, vdim), p[:, 2 * qk + vs:]
+        if rot_dims:
+            q, k = self._turn(q, ctx.positions, table, rot_dims), self._turn(k, ctx.positions, table, rot_dims)
+        k = k * key_scale
+        for r in range(ctx.num_seqs):
+            first, last, slot = ctx.host_q_start[r], ctx.host_q_start[r + 1], ctx.host_seq_slots[r]
+            S = state[slot].view(heads, dim, vdim).clone()
+            for t in range(first, last):
+                S = decay.float()[:, None, None] * S + k[t][:, :, None] * v[t][:, None, :]
+                o = torch.einsum("hdv,hd->hv", S, q[t])
+                o = o * torch.rsqrt((o * o).mean(-1, keepdim=True) + eps)
+                gate = g[t]
+                out[t] = (o.reshape(-1) * gate * torch.sigmoid(gate)).to(out.dtype)
+            state[slot] = S.reshape(-1)
+
+    def scaled_sum(self, a, scale_a, b, scale_b, out):
+        out.copy_((a.float() * scale_a + b.float() * scale_b).to(out.dtype))
+
+    def gated_linear_scan(self, u, gates, gate_bias, rate, xy, blocks, state, taps, ctx, out):
+        tokens, width = u.shape
+        bw = width // blocks
+        z = gates.float() + gate_bias[None]
+        r = torch.sigmoid(z[..., :bw]).reshape(tokens, width)
+        i = torch.sigmoid(z[..., bw:]).reshape(tokens, width)
+        a = torch.exp(rate * r)
+        fed = torch.sqrt(1.0 - a * a) * i * u.float()
+        y = xy[:, width:].float()
+        y = 0.5 * y * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (y + 0.044715 * y ** 3)))
+        for s in range(ctx.num_seqs):
+            first, last, slot = ctx.host_q_start[s], ctx.host_q_start[s + 1], ctx.host_seq_slots[s]
+            S = state[slot, :width].clone()
+            for t in range(first, last):
+                S = a[t] * S + fed[t]
+                out[t] = (S * y[t]).to(out.dtype)
+            state[slot, :width] = S
+
+    def route_chosen(self, logits, gates, experts, top):
+        values, chosen = logits[:, :experts].topk(top, dim=-1)
+        gates.zero_()
+        gates[:, :experts].scatter_(1, chosen, values.softmax(-1))
+        if logits.shape[1] > experts:
+            gates[:, experts:] = torch.sigmoid(logits[:, experts:])
+
+    def gate_silu_mul(self, gate_up, gates, act, experts, ff):
+        columns = act.shape[1]
+        g, u = gate_up[:, :columns].float(), gate_up[:, columns:].float()
+        weight = gates[:, :experts].repeat_interleave(ff, dim=1)
+        if columns > experts * ff:
+            weight = torch.cat((weight, gates[:, experts:experts + 1].expand(-1, columns - experts * ff)), dim=1)
+        act.copy_((weight * (g * torch.sigmoid(g) * u)).to(act.dtype))
 
     # ---- sampling -----------------------------------------------------------------------------------------
     def sample(self, logits, temperature, seeds, draws, out):
