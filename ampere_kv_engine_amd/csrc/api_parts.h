@@ -18,10 +18,50 @@ int akv_embed_pairs(const int* ids, const void* table, const void* pairs, int dt
 int akv_note_fed_tokens(const int* ids, const int* q_start, const int* seq_slots, int* slot_words, int seqs,
                         hipStream_t stream);
 // stream [tokens, hidden] float32.  With `delta` (dtype): stream += delta / rms(delta) * post_weight (or += delta where
-// post_weight is null).  With `out` (dtype): out = stream / rms(stream) * pre_weight, rounded once.
+// post_weight is null: stream += delta_scale * delta).  With `out` (dtype): out = stream / rms(stream) * pre_weight,
+// rounded once.
 int akv_norm_add_norm(float* stream_buf, const void* delta, const float* post_weight, float post_eps,
                       const float* pre_weight, float pre_eps, void* out, int dtype, int tokens, int hidden,
-                      hipStream_t stream);
+                      float delta_scale, hipStream_t stream);
+
+// out = a * scale_a + b * scale_b (float32 arithmetic, one rounding)
+int akv_scaled_sum(const void* a, float scale_a, const void* b, float scale_b, void* out, int dtype, long count,
+                   hipStream_t stream);
+
+// ---- attention with unit-normed queries and keys, softcap, chunks, sink and a gate per head (gated_attention.hip) ------
+// projected [tokens, stride]: rows [q (q_heads x dim) | k (kv_heads x dim) | v (kv_heads x vdim) | ...].  Queries divided
+// by their root mean square per head (where `normed`) go to q_out [tokens, q_heads, dim]; with `slot_map` the keys, the
+// same way, and the values go to the token's slot of the pages: keys [pages, kv_heads, page, dim], values [pages,
+// kv_heads, vdim, page].
+int akv_unit_norm_write(const void* projected, long stride, int dtype, long tokens, int q_heads, int kv_heads, int dim,
+                        int vdim, float eps, int normed, const int* slot_map, void* k_pages, void* v_pages, int page_size,
+                        long num_pages, void* q_out, hipStream_t stream);
+// out [tokens, q_heads, vdim].  score = (q . k) * scale, then softcap * tanh(score / softcap) where softcap > 0; a query at
+// position p sees the keys j <= p with j > p - window (window > 0) and floor(j / chunk) = floor(p / chunk) (chunk > 0);
+// with `sink` the softmax's denominator has one more term exp(0); with `gates` head h's output is multiplied by
+// sigmoid(gates[t * gate_stride + gate_at + h]).
+int akv_gated_attention_rows(const void* q, const void* k_pages, const void* v_pages, const void* gates, long gate_stride,
+                             int gate_at, const int* seq_of_token, const int* positions, const int* block_table,
+                             const int* table_rows, int table_width, void* out, int dtype, long tokens, int q_heads,
+                             int kv_heads, int dim, int vdim, int page_size, long num_pages, float scale, float softcap,
+                             int chunk, int window, int sink, hipStream_t stream);
+
+// ---- mixers with a state of fixed size (recurrent_mixers.hip) ----------------------------------------------------------
+// projected [tokens, stride]: rows [q | k (heads x dim each) | v | g (heads x vdim each)].  q and k are rotated over their
+// first rot_dims dimensions (pairs i, i + rot_dims / 2; `table` [positions, rot_dims / 2, 2] holds cos and sin), k times
+// key_scale; per request and head S [dim, vdim] (at state[slot * state_stride + head * dim * vdim]) <- decay S + k v^T,
+// o = S^T q; out [tokens, heads, vdim] = o / rms(o) * silu(g).
+int akv_retention(const void* projected, long stride, int dtype, int seqs, int heads, int dim, int vdim, int rot_dims,
+                  const float* table, int table_positions, float key_scale, const float* decay, float eps, float* state,
+                  long state_stride, const int* q_start, const int* seq_slots, const int* positions, void* out,
+                  hipStream_t stream);
+// u [tokens, channels]; gates [tokens, blocks, 2 * channels / blocks] float32 (a block's recurrence-gate logits, then its
+// input-gate logits) before their biases `gate_bias` [blocks, 2 * channels / blocks]; a = exp(rate[c] * sigmoid(.));
+// S [channels] at the start of a slot's state <- a S + sqrt(1 - a^2) sigmoid(.) u; out = S * gelu_tanh(y), y at
+// `y_stride` per token.
+int akv_gated_linear_scan(const void* u, int dtype, const float* gates, const float* gate_bias, const float* rate,
+                          const void* y, long y_stride, int seqs, int channels, int blocks, float* state,
+                          long state_stride, const int* q_start, const int* seq_slots, void* out, hipStream_t stream);
 
 // ---- attention over a compressed latent (latent_attention.hip) ------------------------------------------------------
 // down [tokens, q_rank (+ kv_rank + rot)]: q latent normed into `cq`; with `records`: the kv latent normed and the
@@ -60,10 +100,14 @@ int akv_latent_attend_mfma(const void* q_abs, const void* records, const void* l
 
 // ---- selective scan (selective_scan.hip) ----------------------------------------------------------------------------
 // x [tokens, channels] at `x_stride` per token; state [slots, state_stride] float32 holds (taps - 1) x channels at
-// `conv_at`.  out = silu(conv + bias).
+// `conv_at`.  out = silu(conv + bias); akv_conv_taps with `activation` 0: out = conv + bias, 1: silu of it.
 int akv_conv_silu(const void* x, long x_stride, int dtype, const void* weight, const void* bias, int w_dtype,
                   const float* state, long state_stride, long conv_at, const int* seq_of_token, const int* q_start,
                   const int* seq_slots, void* out, int tokens, int channels, int taps, hipStream_t stream);
+int akv_conv_taps(const void* x, long x_stride, int dtype, const void* weight, const void* bias, int w_dtype,
+                  const float* state, long state_stride, long conv_at, const int* seq_of_token, const int* q_start,
+                  const int* seq_slots, void* out, int tokens, int channels, int taps, int activation,
+                  hipStream_t stream);
 int akv_conv_state_update(const void* x, long x_stride, int dtype, float* state, long state_stride, long conv_at,
                           const int* q_start, const int* seq_slots, int seqs, int channels, int taps,
                           hipStream_t stream);
@@ -78,6 +122,12 @@ int akv_selective_scan(const void* x, int dtype, float* dt, const float* bc, con
 // logits [tokens, experts] float32 -> gates [tokens, experts] float32: the softmax score of the chosen experts, 0 elsewhere
 int akv_route(const float* logits, float* gates, int tokens, int experts, int top, int groups, int keep,
               hipStream_t stream);
+// logits [tokens, scored] -> gates: the `top` largest of the first `experts` logits get the softmax over themselves, the
+// other experts 0, every further column its sigmoid
+int akv_route_chosen(const float* logits, float* gates, int tokens, int experts, int scored, int top, hipStream_t stream);
+// act[t, c] = gates[t, e(c)] * silu(gate_up[t, c]) * gate_up[t, columns + c]; e(c) = c / ff below experts * ff, else `experts`
+int akv_gate_silu_mul(const void* gate_up, const float* gates, void* act, int dtype, long tokens, int experts, int ff,
+                      int columns, int scored, hipStream_t stream);
 // act[t, e * ff + j] = gates[t, e] * relu(up[t, e * ff + j])^2
 int akv_gate_relu_squared(const void* up, const float* gates, void* act, int dtype, long tokens, int experts, int ff,
                           hipStream_t stream);

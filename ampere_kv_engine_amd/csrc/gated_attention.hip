@@ -1,0 +1,186 @@
+// Grouped-query attention for designs whose scores and weights are float32 and whose keys and values may differ in
+// width: unit norm of queries and keys with the cache write, and the attention itself with an optional softcap on the
+// scores, chunks of positions, a window, a sink in the softmax's denominator and a gate per head.
+//
+// Keys lie [pages, kv_heads, page, dim], values [pages, kv_heads, vdim, page].  `gated_attention_rows` is the plain path:
+// one wave per (token, query head); keys are visited in tiles of 64 aligned to absolute key positions, so the order of
+// every sum depends on the token's own position only - not on how the request was cut into steps or on what else is in
+// the batch.  Scores, the softmax and the weighted sum are float32.
+
+#include "common.h"
+#include "api_parts.h"
+
+using namespace akv;
+
+namespace {
+
+__device__ __forceinline__ void wave_sync_lds() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// One wave per (token, item): the token's query heads (normed into q_out), its key heads (normed into the token's slot
+// of the key pages) and its value heads (copied into the value pages).  projected rows: [q | k | v | ...].
+template <typename T>
+__global__ __launch_bounds__(256) void unit_norm_write_kernel(const T* __restrict__ projected, long stride, long tokens,
+                                                              int q_heads, int kv_heads, int dim, int vdim, float eps,
+                                                              int normed, const int* __restrict__ slot_map,
+                                                              T* __restrict__ k_pages, T* __restrict__ v_pages, int page_size,
+                                                              long num_pages, T* __restrict__ q_out) {
+  const int waves = blockDim.x / kWave, wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
+  const int items = q_heads + 2 * kv_heads;
+  const long item = static_cast<long>(blockIdx.x) * waves + wave;
+  if (item >= tokens * items) return;
+  const long n = item / items;
+  const int which = static_cast<int>(item % items);
+  const T* row = projected + n * stride;
+  if (which < q_heads + kv_heads) {
+    const bool is_q = which < q_heads;
+    const T* x = row + static_cast<long>(which) * dim;       // (key heads follow the query heads at the same width)
+    T* y;
+    if (is_q) {
+      y = q_out + (n * q_heads + which) * dim;
+    } else {
+      if (slot_map == nullptr) return;
+      const long slot = slot_map[n];
+      const long page = slot / page_size;
+      if (slot < 0 || page >= num_pages) return;
+      y = k_pages + ((page * kv_heads + (which - q_heads)) * page_size + slot % page_size) * dim;
+    }
+    float squares = 0.f;
+    for (int i = lane; i < dim; i += kWave) {
+      const float v = to_float(x[i]);
+      squares += v * v;
+    }
+    const float scale = normed ? rsqrtf(wave_sum(squares) / static_cast<float>(dim) + eps) : 1.f;
+    for (int i = lane; i < dim; i += kWave) y[i] = from_float<T>(to_float(x[i]) * scale);
+  } else {
+    if (slot_map == nullptr) return;
+    const int h = which - q_heads - kv_heads;
+    const long slot = slot_map[n];
+    const long page = slot / page_size;
+    if (slot < 0 || page >= num_pages) return;
+    const T* x = row + static_cast<long>(q_heads + kv_heads) * dim + static_cast<long>(h) * vdim;
+    T* y = v_pages + (page * kv_heads + h) * vdim * page_size + slot % page_size;
+    for (int i = lane; i < vdim; i += kWave) y[static_cast<long>(i) * page_size] = x[i];
+  }
+}
+
+constexpr int kMaxValueRegs = 4;  // value widths up to 256: each lane owns dims lane, lane + 64, ...
+
+template <typename T>
+__global__ __launch_bounds__(256) void gated_attention_rows_kernel(
+    const T* __restrict__ q, const T* __restrict__ k_pages, const T* __restrict__ v_pages, const T* __restrict__ gates,
+    long gate_stride, int gate_at, const int* __restrict__ seq_of_token, const int* __restrict__ positions,
+    const int* __restrict__ block_table, const int* __restrict__ table_rows, int table_width, T* __restrict__ out,
+    long tokens, int q_heads, int kv_heads, int dim, int vdim, int page_size, long num_pages, float scale, float softcap,
+    int chunk, int window, int sink) {
+  extern __shared__ unsigned char lds_raw[];
+  const int waves = blockDim.x / kWave, wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
+  const long row = static_cast<long>(blockIdx.x) * waves + wave;
+  if (row >= tokens * q_heads) return;
+  const size_t per_wave = (static_cast<size_t>(dim) * 4 + kWave * 4 + kWave * 8 + 7) / 8 * 8;
+  float* qs = reinterpret_cast<float*>(lds_raw + wave * per_wave);
+  float* ps = qs + dim;
+  long* offs = reinterpret_cast<long*>(lds_raw + wave * per_wave + (static_cast<size_t>(dim) * 4 + kWave * 4 + 7) / 8 * 8);
+
+  const long n = row / q_heads;
+  const int h = static_cast<int>(row % q_heads);
+  const int kvh = h / (q_heads / kv_heads);
+  const int r = table_rows != nullptr ? table_rows[seq_of_token[n]] : seq_of_token[n];
+  const int pos = positions[n];
+  int lowest = window > 0 ? max(0, pos - window + 1) : 0;
+  if (chunk > 0) lowest = max(lowest, pos / chunk * chunk);
+  for (int i = lane; i < dim; i += kWave) qs[i] = to_float(q[row * dim + i]);
+  wave_sync_lds();
+
+  // with a sink the sums start as if a key of score 0 and no value had been seen
+  float m = sink ? 0.f : -INFINITY, l = sink ? 1.f : 0.f;
+  float acc[kMaxValueRegs] = {0.f, 0.f, 0.f, 0.f};
+  for (int tile = lowest / kWave; tile * kWave <= pos; ++tile) {
+    const int j = tile * kWave + lane;
+    const bool valid = j >= lowest && j <= pos;
+    float s = -INFINITY;
+    long value_at = -1;
+    if (valid) {
+      const long page = block_table[static_cast<long>(r) * table_width + j / page_size];
+      if (page < 0 || page >= num_pages) {
+        s = __uint_as_float(0x7fc00000u);  // a page that is not the request's: poison, never read
+      } else {
+        const T* kp = k_pages + ((page * kv_heads + kvh) * page_size + j % page_size) * dim;
+        float dot = 0.f;
+        for (int i = 0; i < dim; ++i) dot = fmaf(qs[i], to_float(kp[i]), dot);
+        s = dot * scale;
+        if (softcap > 0.f) s = softcap * tanhf(s / softcap);
+        value_at = (page * kv_heads + kvh) * vdim * page_size + j % page_size;  // values are [vdim, page_size]
+      }
+    }
+    const float m_new = fmaxf(m, wave_max(s));
+    const float p = valid ? expf(s - m_new) : 0.f;
+    const float correction = expf(m - m_new);
+    l = l * correction + wave_sum(p);
+    m = m_new;
+    ps[lane] = p;
+    offs[lane] = value_at;
+    wave_sync_lds();
+#pragma unroll
+    for (int c = 0; c < kMaxValueRegs; ++c) acc[c] *= correction;
+    for (int jj = 0; jj < kWave; ++jj) {
+      const long at = offs[jj];
+      if (at < 0) continue;  // uniform over the wave
+      const float pj = ps[jj];
+#pragma unroll
+      for (int c = 0; c < kMaxValueRegs; ++c) {
+        const int i = lane + c * kWave;
+        if (i < vdim) acc[c] = fmaf(pj, to_float(v_pages[at + static_cast<long>(i) * page_size]), acc[c]);
+      }
+    }
+    wave_sync_lds();
+  }
+  float gate = 1.f;
+  if (gates != nullptr) gate = 1.f / (1.f + expf(-to_float(gates[n * gate_stride + gate_at + h])));
+#pragma unroll
+  for (int c = 0; c < kMaxValueRegs; ++c) {
+    const int i = lane + c * kWave;
+    if (i < vdim) out[row * vdim + i] = from_float<T>(acc[c] / l * gate);
+  }
+}
+
+}  // namespace
+
+extern "C" {
+
+int akv_unit_norm_write(const void* projected, long stride, int dtype, long tokens, int q_heads, int kv_heads, int dim,
+                        int vdim, float eps, int normed, const int* slot_map, void* k_pages, void* v_pages, int page_size,
+                        long num_pages, void* q_out, hipStream_t stream) {
+  if (tokens <= 0) return 0;
+  if (q_heads <= 0 || kv_heads <= 0 || dim <= 0 || vdim <= 0 || page_size <= 0) return -2;
+  const long items = tokens * (q_heads + 2 * kv_heads);
+  AKV_DISPATCH(dtype, T, unit_norm_write_kernel<T><<<static_cast<unsigned>((items + 3) / 4), 256, 0, stream>>>(
+                             static_cast<const T*>(projected), stride, tokens, q_heads, kv_heads, dim, vdim, eps, normed,
+                             slot_map, static_cast<T*>(k_pages), static_cast<T*>(v_pages), page_size, num_pages,
+                             static_cast<T*>(q_out)));
+  return AKV_LAUNCH_STATUS();
+}
+
+int akv_gated_attention_rows(const void* q, const void* k_pages, const void* v_pages, const void* gates, long gate_stride,
+                             int gate_at, const int* seq_of_token, const int* positions, const int* block_table,
+                             const int* table_rows, int table_width, void* out, int dtype, long tokens, int q_heads,
+                             int kv_heads, int dim, int vdim, int page_size, long num_pages, float scale, float softcap,
+                             int chunk, int window, int sink, hipStream_t stream) {
+  if (tokens <= 0) return 0;
+  if (vdim > kMaxValueRegs * kWave || dim <= 0 || q_heads % kv_heads != 0) return -2;
+  const long rows = tokens * q_heads;
+  const size_t per_wave = (static_cast<size_t>(dim) * 4 + kWave * 4 + kWave * 8 + 7) / 8 * 8;
+  const size_t lds = 4 * per_wave;
+  if (lds > 64 * 1024) return -2;
+  AKV_DISPATCH(dtype, T,
+               gated_attention_rows_kernel<T><<<static_cast<unsigned>((rows + 3) / 4), 256, lds, stream>>>(
+                   static_cast<const T*>(q), static_cast<const T*>(k_pages), static_cast<const T*>(v_pages),
+                   static_cast<const T*>(gates), gate_stride, gate_at, seq_of_token, positions, block_table, table_rows,
+                   table_width, static_cast<T*>(out), tokens, q_heads, kv_heads, dim, vdim, page_size, num_pages, scale,
+                   softcap, chunk, window, sink));
+  return AKV_LAUNCH_STATUS();
+}
+}

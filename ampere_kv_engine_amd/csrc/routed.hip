@@ -112,9 +112,114 @@ __global__ void gate_relu_squared_by8_kernel(const bf16_t* __restrict__ up, cons
   *reinterpret_cast<uint4*>(act + index) = packed;
 }
 
+// One wave per token: the `top` experts with the largest logits (equal logits go to the lower index) are chosen and
+// weighted by the softmax over their logits alone; every other expert's gate is an exact zero.  A row may hold further
+// logits after the experts' (`scored` in all): each of those becomes its own sigmoid - the gate of an expert that every
+// token uses.
+__global__ __launch_bounds__(256) void route_chosen_kernel(const float* __restrict__ logits, float* __restrict__ gates,
+                                                           int tokens, int experts, int scored, int top) {
+  extern __shared__ float lds[];
+  const int waves = blockDim.x / kWave, wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
+  const int n = blockIdx.x * waves + wave;
+  if (n >= tokens) return;
+  float* score = lds + static_cast<size_t>(wave) * (experts + 2 * top);   // [experts], -inf once chosen
+  float* chosen_value = score + experts;                                  // [top]
+  float* chosen_index = chosen_value + top;                               // [top]
+  const float* row = logits + static_cast<size_t>(n) * scored;
+  float* gate_row = gates + static_cast<size_t>(n) * scored;
+  for (int e = lane; e < scored; e += kWave) {
+    if (e < experts) {
+      score[e] = row[e];
+      gate_row[e] = 0.f;
+    } else {
+      gate_row[e] = 1.f / (1.f + expf(-row[e]));
+    }
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  for (int k = 0; k < top; ++k) {
+    float best = -INFINITY;
+    int at = 0x7fffffff;
+    for (int e = lane; e < experts; e += kWave) {
+      const float z = score[e];
+      if (z > best) {          // (ascending e: the lower index keeps an equal score)
+        best = z;
+        at = e;
+      }
+    }
+#pragma unroll
+    for (int offset = kWave / 2; offset > 0; offset >>= 1) {
+      const float other = __shfl_xor(best, offset, kWave);
+      const int other_at = __shfl_xor(at, offset, kWave);
+      if (other > best || (other == best && other_at < at)) {
+        best = other;
+        at = other_at;
+      }
+    }
+    if (at == 0x7fffffff) at = 0;     // (nothing finite left: cannot happen while top <= experts and logits are finite)
+    if (lane == 0) {
+      chosen_value[k] = best;
+      chosen_index[k] = static_cast<float>(at);
+      score[at] = -INFINITY;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  }
+  if (lane == 0) {
+    const float highest = chosen_value[0];     // the first chosen is the largest
+    float total = 0.f;
+    for (int k = 0; k < top; ++k) total += expf(chosen_value[k] - highest);
+    for (int k = 0; k < top; ++k) gate_row[static_cast<int>(chosen_index[k])] = expf(chosen_value[k] - highest) / total;
+  }
+}
+
+// act[t, c] = gates[t, e(c)] * silu(gate_up[t, c]) * gate_up[t, columns + c]: the experts' gate rows first, then their up
+// rows; column c belongs to expert c / ff while c < experts * ff and to the expert every token uses beyond (gate number
+// `experts`).  Float32 up to the one rounding; an expert that was not chosen gives exact zeros.
+template <typename T>
+__global__ void gate_silu_mul_kernel(const T* __restrict__ gate_up, const float* __restrict__ gates, T* __restrict__ act,
+                                     long tokens, int experts, int ff, int columns, int scored) {
+  const long index = static_cast<long>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (index >= tokens * columns) return;
+  const long n = index / columns;
+  const int c = static_cast<int>(index % columns);
+  const int e = c < experts * ff ? c / ff : experts;
+  const float g = gates[n * scored + e];
+  float value = 0.f;
+  if (g != 0.f) {
+    const float z = to_float(gate_up[n * 2 * columns + c]);
+    value = g * (z / (1.f + expf(-z)) * to_float(gate_up[n * 2 * columns + columns + c]));
+  }
+  act[index] = from_float<T>(value);
+}
+
 }  // namespace
 
 extern "C" {
+
+int akv_route_chosen(const float* logits, float* gates, int tokens, int experts, int scored, int top, hipStream_t stream) {
+  if (tokens <= 0) return 0;
+  if (experts <= 0 || top <= 0 || top > experts || scored < experts) return -2;
+  const int waves = 4;
+  const size_t lds_bytes = static_cast<size_t>(waves) * (experts + 2 * top) * 4;
+  if (lds_bytes > 64 * 1024) return -2;
+  route_chosen_kernel<<<(tokens + waves - 1) / waves, waves * kWave, lds_bytes, stream>>>(logits, gates, tokens, experts,
+                                                                                          scored, top);
+  return AKV_LAUNCH_STATUS();
+}
+
+int akv_gate_silu_mul(const void* gate_up, const float* gates, void* act, int dtype, long tokens, int experts, int ff,
+                      int columns, int scored, hipStream_t stream) {
+  const long count = tokens * columns;
+  if (count <= 0) return 0;
+  if (columns < experts * ff || scored < experts + (columns > experts * ff ? 1 : 0)) return -2;
+  AKV_DISPATCH(dtype, T, gate_silu_mul_kernel<T><<<static_cast<unsigned>((count + 255) / 256), 256, 0, stream>>>(
+                             static_cast<const T*>(gate_up), gates, static_cast<T*>(act), tokens, experts, ff, columns,
+                             scored));
+  return AKV_LAUNCH_STATUS();
+}
 
 int akv_route(const float* logits, float* gates, int tokens, int experts, int top, int groups, int keep,
               hipStream_t stream) {

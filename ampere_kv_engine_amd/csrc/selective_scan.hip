@@ -16,7 +16,7 @@ __device__ __forceinline__ float silu(float v) { return v / (1.f + expf(-v)); }
 __device__ __forceinline__ float softplus(float v) { return v > 20.f ? v : log1pf(expf(v)); }
 
 // ---- convolution over the portion and what the slot remembers of the tokens before it --------------------------------
-template <typename T, typename TW>
+template <typename T, typename TW, bool SILU>
 __global__ __launch_bounds__(256) void conv_silu_kernel(const T* __restrict__ x, long x_stride, const TW* __restrict__ weight,
                                                         const TW* __restrict__ bias, const float* __restrict__ state,
                                                         long state_stride, long conv_at,
@@ -41,7 +41,7 @@ __global__ __launch_bounds__(256) void conv_silu_kernel(const T* __restrict__ x,
     }
     acc = fmaf(to_float(weight[static_cast<long>(c) * taps + k]), v, acc);
   }
-  out[static_cast<long>(n) * channels + c] = from_float<T>(silu(acc));
+  out[static_cast<long>(n) * channels + c] = from_float<T>(SILU ? silu(acc) : acc);
 }
 
 // After the convolution has read the old inputs: the slot keeps the last taps - 1 of (old inputs, the portion's).
@@ -193,18 +193,31 @@ extern "C" {
 int akv_conv_silu(const void* x, long x_stride, int dtype, const void* weight, const void* bias, int w_dtype,
                   const float* state, long state_stride, long conv_at, const int* seq_of_token, const int* q_start,
                   const int* seq_slots, void* out, int tokens, int channels, int taps, hipStream_t stream) {
+  return akv_conv_taps(x, x_stride, dtype, weight, bias, w_dtype, state, state_stride, conv_at, seq_of_token, q_start,
+                       seq_slots, out, tokens, channels, taps, 1, stream);
+}
+
+int akv_conv_taps(const void* x, long x_stride, int dtype, const void* weight, const void* bias, int w_dtype,
+                  const float* state, long state_stride, long conv_at, const int* seq_of_token, const int* q_start,
+                  const int* seq_slots, void* out, int tokens, int channels, int taps, int activation,
+                  hipStream_t stream) {
   if (tokens <= 0) return 0;
-  if (taps < 1 || channels <= 0) return -2;
+  if (taps < 1 || channels <= 0 || activation < 0 || activation > 1) return -2;
   const dim3 grid(tokens, (channels + 255) / 256);
-#define AKV_CONV(T, TW)                                                                                            \
-  conv_silu_kernel<T, TW><<<grid, 256, 0, stream>>>(static_cast<const T*>(x), x_stride, static_cast<const TW*>(weight), \
-                                                    static_cast<const TW*>(bias), state, state_stride, conv_at,     \
-                                                    seq_of_token, q_start, seq_slots, static_cast<T*>(out), channels, taps)
+#define AKV_CONV_ARGS(T, TW)                                                                                         \
+  static_cast<const T*>(x), x_stride, static_cast<const TW*>(weight), static_cast<const TW*>(bias), state, state_stride, \
+      conv_at, seq_of_token, q_start, seq_slots, static_cast<T*>(out), channels, taps
+#define AKV_CONV(T, TW)                                                                          \
+  do {                                                                                           \
+    if (activation == 1) conv_silu_kernel<T, TW, true><<<grid, 256, 0, stream>>>(AKV_CONV_ARGS(T, TW)); \
+    else conv_silu_kernel<T, TW, false><<<grid, 256, 0, stream>>>(AKV_CONV_ARGS(T, TW));           \
+  } while (0)
   if (dtype == kF32 && w_dtype == kF32) AKV_CONV(float, float);
   else if (dtype == kBF16 && w_dtype == kBF16) AKV_CONV(bf16_t, bf16_t);
   else if (dtype == kBF16 && w_dtype == kF32) AKV_CONV(bf16_t, float);
   else return -1;
 #undef AKV_CONV
+#undef AKV_CONV_ARGS
   return AKV_LAUNCH_STATUS();
 }
 

@@ -77,7 +77,7 @@ template <typename T, int GROUPS>
 __global__ __launch_bounds__(256) void norm_add_norm_rows_kernel(float* __restrict__ stream, const T* __restrict__ delta,
                                                                  const float* __restrict__ post_weight, float post_eps,
                                                                  const float* __restrict__ pre_weight, float pre_eps,
-                                                                 T* __restrict__ out, int hidden) {
+                                                                 T* __restrict__ out, int hidden, float delta_scale) {
   __shared__ float scratch[16];
   const size_t base = static_cast<size_t>(blockIdx.x) * hidden;
   float4 kept[GROUPS], added[GROUPS];
@@ -107,6 +107,8 @@ __global__ __launch_bounds__(256) void norm_add_norm_rows_kernel(float* __restri
       if (post_weight != nullptr) {
         const float4 w = read4<float>(post_weight + i);
         d = make_float4(d.x * post_scale * w.x, d.y * post_scale * w.y, d.z * post_scale * w.z, d.w * post_scale * w.w);
+      } else {
+        d = make_float4(d.x * delta_scale, d.y * delta_scale, d.z * delta_scale, d.w * delta_scale);
       }
       kept[j] = make_float4(kept[j].x + d.x, kept[j].y + d.y, kept[j].z + d.z, kept[j].w + d.w);
       write4<float>(stream + base + i, kept[j]);
@@ -131,7 +133,7 @@ template <typename T>
 __global__ __launch_bounds__(256) void norm_add_norm_kernel(float* __restrict__ stream, const T* __restrict__ delta,
                                                             const float* __restrict__ post_weight, float post_eps,
                                                             const float* __restrict__ pre_weight, float pre_eps,
-                                                            T* __restrict__ out, int hidden) {
+                                                            T* __restrict__ out, int hidden, float delta_scale) {
   __shared__ float scratch[16];
   const size_t base = static_cast<size_t>(blockIdx.x) * hidden;
   float* s = stream + base;
@@ -148,7 +150,7 @@ __global__ __launch_bounds__(256) void norm_add_norm_kernel(float* __restrict__ 
       post_scale = rsqrtf(block_sum(acc, scratch) / static_cast<float>(hidden) + post_eps);
     }
     for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
-      const float add = post_weight != nullptr ? to_float(d[i]) * post_scale * post_weight[i] : to_float(d[i]);
+      const float add = post_weight != nullptr ? to_float(d[i]) * post_scale * post_weight[i] : to_float(d[i]) * delta_scale;
       const float v = s[i] + add;
       s[i] = v;
       squares += v * v;
@@ -166,9 +168,24 @@ __global__ __launch_bounds__(256) void norm_add_norm_kernel(float* __restrict__ 
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) o[i] = from_float<T>(s[i] * scale * pre_weight[i]);
 }
 
+// out = a * scale_a + b * scale_b, formed in float32 and rounded once (out may be a or b).
+template <typename T>
+__global__ void scaled_sum_kernel(const T* a, float scale_a, const T* b, float scale_b, T* out, long count) {
+  const long index = static_cast<long>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (index < count) out[index] = from_float<T>(to_float(a[index]) * scale_a + to_float(b[index]) * scale_b);
+}
+
 }  // namespace
 
 extern "C" {
+
+int akv_scaled_sum(const void* a, float scale_a, const void* b, float scale_b, void* out, int dtype, long count,
+                   hipStream_t stream) {
+  if (count <= 0) return 0;
+  AKV_DISPATCH(dtype, T, scaled_sum_kernel<T><<<static_cast<unsigned>((count + 255) / 256), 256, 0, stream>>>(
+                             static_cast<const T*>(a), scale_a, static_cast<const T*>(b), scale_b, static_cast<T*>(out), count));
+  return AKV_LAUNCH_STATUS();
+}
 
 int akv_parts_slot_layout(int* out) {
   out[0] = kSlotWords;
@@ -197,10 +214,10 @@ int akv_note_fed_tokens(const int* ids, const int* q_start, const int* seq_slots
 
 int akv_norm_add_norm(float* stream_buf, const void* delta, const float* post_weight, float post_eps,
                       const float* pre_weight, float pre_eps, void* out, int dtype, int tokens, int hidden,
-                      hipStream_t stream) {
+                      float delta_scale, hipStream_t stream) {
   if (tokens <= 0) return 0;
   if (out != nullptr && pre_weight == nullptr) return -2;
-#define AKV_NORM_ARGS stream_buf, static_cast<const T*>(delta), post_weight, post_eps, pre_weight, pre_eps, static_cast<T*>(out), hidden
+#define AKV_NORM_ARGS stream_buf, static_cast<const T*>(delta), post_weight, post_eps, pre_weight, pre_eps, static_cast<T*>(out), hidden, delta_scale
   AKV_DISPATCH(dtype, T, {
     if (hidden % 4 == 0 && hidden >= 4 && hidden <= 256 * 4 * 2) norm_add_norm_rows_kernel<T, 2><<<tokens, 256, 0, stream>>>(AKV_NORM_ARGS);
     else if (hidden % 4 == 0 && hidden <= 256 * 4 * 8) norm_add_norm_rows_kernel<T, 8><<<tokens, 256, 0, stream>>>(AKV_NORM_ARGS);

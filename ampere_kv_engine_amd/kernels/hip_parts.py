@@ -39,7 +39,9 @@ class PartsKernels:
             for name in ("akv_embed_pairs", "akv_note_fed_tokens", "akv_norm_add_norm", "akv_latent_encode",
                          "akv_rotate_queries", "akv_heads_linear", "akv_latent_attend", "akv_latent_attend_mfma", "akv_conv_silu",
                          "akv_conv_state_update", "akv_selective_scan", "akv_route", "akv_gate_relu_squared",
-                         "akv_parts_slot_layout"):
+                         "akv_parts_slot_layout", "akv_conv_taps", "akv_scaled_sum", "akv_unit_norm_write",
+                         "akv_gated_attention_rows", "akv_retention", "akv_gated_linear_scan", "akv_route_chosen",
+                         "akv_gate_silu_mul"):
                 getattr(lib, name).restype = ctypes.c_int
             layout = (ctypes.c_int * 3)()
             lib.akv_parts_slot_layout(layout)
@@ -94,9 +96,9 @@ class PartsKernels:
         self._check(lib.akv_note_fed_tokens(_ptr(ids), _ptr(ctx.q_start), _ptr(ctx.seq_slots), _ptr(words), ctx.num_seqs,
                                             self._stream()), "note_fed_tokens")
 
-    def norm_add_norm(self, stream, delta, post_weight, post_eps, pre_weight, pre_eps, out) -> None:
-        """stream (float32) += delta / rms(delta) * post_weight (+= delta where `post_weight` is None; nothing where
-        `delta` is None); then, where `out` is given, out = stream / rms(stream) * pre_weight.  Float32 up to the one
+    def norm_add_norm(self, stream, delta, post_weight, post_eps, pre_weight, pre_eps, out, delta_scale: float = 1.0) -> None:
+        """stream (float32) += delta / rms(delta) * post_weight (+= delta_scale * delta where `post_weight` is None; nothing
+        where `delta` is None); then, where `out` is given, out = stream / rms(stream) * pre_weight.  Float32 up to the one
         rounding of a stored result."""
         tokens, hidden = stream.shape
         self._dense(stream, "stream", torch.float32)
@@ -114,7 +116,16 @@ class PartsKernels:
             return
         self._check(self._parts().akv_norm_add_norm(_ptr(stream), _ptr(delta), _ptr(post_weight), ctypes.c_float(post_eps),
                                                     _ptr(pre_weight), ctypes.c_float(pre_eps), _ptr(out), _DTYPE_CODE[dtype],
-                                                    tokens, hidden, self._stream()), "norm_add_norm")
+                                                    tokens, hidden, ctypes.c_float(delta_scale), self._stream()),
+                    "norm_add_norm")
+
+    def scaled_sum(self, a, scale_a: float, b, scale_b: float, out) -> None:
+        """out = a * scale_a + b * scale_b, in float32 with one rounding (`out` may be `a` or `b`)."""
+        self._dense(a, "a")
+        self._dense(b, "b", a.dtype, tuple(a.shape))
+        self._dense(out, "out", a.dtype, tuple(a.shape))
+        self._check(self._parts().akv_scaled_sum(_ptr(a), ctypes.c_float(scale_a), _ptr(b), ctypes.c_float(scale_b), _ptr(out),
+                                                 self._code_of(a), _long(a.numel()), self._stream()), "scaled_sum")
 
     # ---- attention over a compressed latent --------------------------------------------------------------------------
     MATRIX_CORE_LATENTS = (128, 256, 512)
@@ -288,9 +299,9 @@ class PartsKernels:
         if max(ctx.host_seq_slots) >= state.shape[0]:
             self._refuse("a request's slot lies outside the state")
 
-    def conv_silu(self, xz, channels, weight, bias, state, n_state, ctx, out) -> None:
+    def conv_silu(self, xz, channels, weight, bias, state, n_state, ctx, out, activation: str = "silu") -> None:
         """out[t, c] = silu(bias[c] + sum_k weight[c, k] * x[t - (taps - 1 - k), c]) over the first `channels` columns
-        of `xz`; inputs before a portion come from the request's state (zeros before its first token).  Afterwards the
+        of `xz` (with `activation="none"` the sum as it is); inputs before a portion come from the request's state (zeros before its first token).  Afterwards the
         state holds the last taps - 1 inputs of every request of the step."""
         tokens, taps = xz.shape[0], weight.shape[1]
         self._dense(xz, "xz")
@@ -302,10 +313,12 @@ class PartsKernels:
         self._scan_state(state, ctx, channels, n_state, taps)
         self._step_arrays(ctx, tokens)
         lib, conv_at = self._parts(), channels * n_state
-        self._check(lib.akv_conv_silu(_ptr(xz), _long(xz.shape[1]), self._code_of(xz), _ptr(weight), _ptr(bias),
+        if activation not in ("silu", "none"):
+            self._refuse(f"the convolution's activation is 'silu' or 'none', not {activation!r}")
+        self._check(lib.akv_conv_taps(_ptr(xz), _long(xz.shape[1]), self._code_of(xz), _ptr(weight), _ptr(bias),
                                       self._code_of(weight), _ptr(state), _long(state.shape[1]), _long(conv_at),
                                       _ptr(ctx.seq_of_token), _ptr(ctx.q_start), _ptr(ctx.seq_slots), _ptr(out), tokens,
-                                      channels, taps, self._stream()), "conv_silu")
+                                      channels, taps, 1 if activation == "silu" else 0, self._stream()), "conv_taps")
         self._check(lib.akv_conv_state_update(_ptr(xz), _long(xz.shape[1]), self._code_of(xz), _ptr(state),
                                               _long(state.shape[1]), _long(conv_at), _ptr(ctx.q_start), _ptr(ctx.seq_slots),
                                               ctx.num_seqs, channels, taps, self._stream()), "conv_state_update")
@@ -352,3 +365,141 @@ class PartsKernels:
         self._check(self._parts().akv_gate_relu_squared(_ptr(up), _ptr(gates), _ptr(act), self._code_of(up), _long(tokens),
                                                         experts, up.shape[1] // experts, self._stream()),
                     "gate_relu_squared")
+
+    def route_chosen(self, logits, gates, experts: int, top: int) -> None:
+        """gates[t, e] = the softmax over the `top` largest of the first `experts` logits for those experts (equal logits
+        go to the lower index), 0 for the others; every further column of a row becomes its sigmoid."""
+        tokens, scored = logits.shape
+        self._dense(logits, "logits", torch.float32)
+        self._dense(gates, "gates", torch.float32, (tokens, scored))
+        self._check(self._parts().akv_route_chosen(_ptr(logits), _ptr(gates), tokens, experts, scored, top, self._stream()),
+                    "route_chosen")
+
+    def gate_silu_mul(self, gate_up, gates, act, experts: int, ff: int) -> None:
+        """act[t, c] = gates[t, e(c)] * silu(gate_up[t, c]) * gate_up[t, columns + c]; column c belongs to expert c // ff
+        below experts * ff and to the expert every token uses beyond (gate number `experts`)."""
+        tokens, columns = act.shape
+        self._dense(act, "act")
+        self._dense(gate_up, "gate_up", act.dtype, (tokens, 2 * columns))
+        self._dense(gates, "gates", torch.float32)
+        if gates.dim() != 2 or gates.shape[0] != tokens or gates.shape[1] < experts + (1 if columns > experts * ff else 0):
+            self._refuse(f"gates must be [tokens, at least the experts (and the shared one)], got {tuple(gates.shape)}")
+        self._check(self._parts().akv_gate_silu_mul(_ptr(gate_up), _ptr(gates), _ptr(act), self._code_of(act), _long(tokens),
+                                                    experts, ff, columns, gates.shape[1], self._stream()), "gate_silu_mul")
+
+    # ---- attention with unit-normed queries and keys, a softcap, chunks, a sink and a gate per head ----------------------
+    MAX_VALUE_DIM = 256
+
+    def check_gated_attention_sizes(self, q_heads: int, kv_heads: int, dim: int, vdim: int, page_size: int) -> None:
+        if q_heads % kv_heads:
+            self._refuse(f"q_heads {q_heads} is not a multiple of kv_heads {kv_heads}")
+        if not 0 < vdim <= self.MAX_VALUE_DIM or not 0 < dim <= 2048:
+            self._refuse(f"the attention takes values up to {self.MAX_VALUE_DIM} wide and keys up to 2048, not {vdim} and {dim}")
+
+    def _gated_pages(self, k_pages, v_pages, kv_heads, dim, vdim, dtype):
+        self._dense(k_pages, "k_pages", dtype)
+        if k_pages.dim() != 4 or k_pages.shape[1] != kv_heads or k_pages.shape[3] != dim:
+            self._refuse(f"key pages must be [pages, {kv_heads}, page_size, {dim}], got {tuple(k_pages.shape)}")
+        self._dense(v_pages, "v_pages", dtype, (k_pages.shape[0], kv_heads, vdim, k_pages.shape[2]))
+        return k_pages.shape[0], k_pages.shape[2]
+
+    def unit_norm_write(self, projected, q_heads, kv_heads, dim, vdim, eps, slot_map, k_pages, v_pages, q_out) -> None:
+        """projected [tokens, q | k | v | ...]: the query heads divided by their root mean square (eps inside the root;
+        `eps` None: as they are) -> q_out; with `slot_map` the key heads, the same way, and the value heads into the
+        tokens' slots of the pages."""
+        tokens = projected.shape[0]
+        self._dense(projected, "projected")
+        if projected.dim() != 2 or projected.shape[1] < (q_heads + kv_heads) * dim + kv_heads * vdim:
+            self._refuse(f"projected rows must hold queries, keys and values, got {tuple(projected.shape)}")
+        self._dense(q_out, "q_out", projected.dtype, (tokens, q_heads * dim))
+        num_pages, page_size = self._gated_pages(k_pages, v_pages, kv_heads, dim, vdim, projected.dtype)
+        if slot_map is not None:
+            self._dense(slot_map, "slot_map", torch.int32, (tokens,))
+        self._check(self._parts().akv_unit_norm_write(
+            _ptr(projected), _long(projected.shape[1]), self._code_of(projected), _long(tokens), q_heads, kv_heads, dim, vdim,
+            ctypes.c_float(eps if eps is not None else 0.0), 0 if eps is None else 1, _ptr(slot_map), _ptr(k_pages),
+            _ptr(v_pages), page_size, _long(num_pages), _ptr(q_out), self._stream()), "unit_norm_write")
+
+    def gated_attention(self, q, k_pages, v_pages, gates, gate_at, ctx, meta, q_heads, kv_heads, dim, vdim, scale, softcap,
+                        chunk, window, sink, out) -> None:
+        """Every query head attends the keys of its request that it sees (see `parts/gated_attention.py`) -> out
+        [tokens, q_heads * vdim]; `gates` [tokens, width]: head h's output times sigmoid(gates[t, gate_at + h])."""
+        tokens = q.shape[0]
+        self._dense(q, "q", None, (tokens, q_heads * dim))
+        self._dense(out, "out", q.dtype, (tokens, q_heads * vdim))
+        num_pages, page_size = self._gated_pages(k_pages, v_pages, kv_heads, dim, vdim, q.dtype)
+        gate_stride = 0
+        if gates is not None:
+            self._dense(gates, "gates", q.dtype)
+            if gates.dim() != 2 or gates.shape[0] != tokens or gate_at + q_heads > gates.shape[1]:
+                self._refuse(f"gates must be [tokens, at least {gate_at + q_heads}], got {tuple(gates.shape)}")
+            gate_stride = gates.shape[1]
+        self._dense(meta.block_table, "block_table", torch.int32)
+        if meta.block_table.dim() != 2 or meta.block_table.shape[1] != meta.width:
+            self._refuse("the block table does not have the width the step names")
+        self._step_arrays(ctx, tokens)
+        if meta.rows is not None:
+            self._dense(meta.rows, "table rows", torch.int32, (ctx.num_seqs,))
+            if max(ctx.host_seq_slots) >= meta.block_table.shape[0]:
+                self._refuse("a request's slot lies outside the block table")
+        elif ctx.num_seqs > meta.block_table.shape[0]:
+            self._refuse("the block table has fewer rows than the step has requests")
+        if ctx.max_seq_len > meta.width * page_size:
+            self._refuse("a request is longer than its row of the block table")
+        self._check(self._parts().akv_gated_attention_rows(
+            _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(gates), _long(gate_stride), gate_at, _ptr(ctx.seq_of_token),
+            _ptr(ctx.positions), _ptr(meta.block_table), _ptr(meta.rows), meta.width, _ptr(out), self._code_of(q),
+            _long(tokens), q_heads, kv_heads, dim, vdim, page_size, _long(num_pages), ctypes.c_float(scale),
+            ctypes.c_float(softcap if softcap is not None else 0.0), int(chunk) if chunk is not None else 0,
+            int(window) if window is not None else 0, 1 if sink else 0, self._stream()), "gated_attention")
+
+    # ---- mixers with a state of fixed size -----------------------------------------------------------------------------
+    def check_retention_sizes(self, heads: int, dim: int, vdim: int) -> None:
+        if not 0 < vdim <= 1024 or dim <= 0 or vdim * ((dim + 63) // 64) > 1024:
+            self._refuse(f"retention keeps a head's state [{dim}, {vdim}] in one block's registers: up to 65,536 values")
+
+    def retention(self, projected, heads, dim, vdim, rot_dims, table, key_scale, decay, eps, state, ctx, out) -> None:
+        """projected [tokens, q | k | v | g] -> out [tokens, heads * vdim] = (S^T q) / rms * silu(g) with S <- decay S +
+        k v^T per request and head (see `parts/retention.py`); S lies in the request's slot of `state`, float32."""
+        tokens = projected.shape[0]
+        self._dense(projected, "projected", None, (tokens, 2 * heads * (dim + vdim)))
+        self._dense(out, "out", projected.dtype, (tokens, heads * vdim))
+        self._dense(decay, "decay", torch.float32, (heads,))
+        self._dense(state, "state", torch.float32)
+        if state.dim() != 2 or state.shape[1] != heads * dim * vdim:
+            self._refuse(f"retention's state must be [slots, {heads * dim * vdim}], got {tuple(state.shape)}")
+        if max(ctx.host_seq_slots) >= state.shape[0]:
+            self._refuse("a request's slot lies outside the state")
+        positions = 0
+        if rot_dims:
+            self._dense(table, "table", torch.float32)
+            if table.dim() != 3 or table.shape[1] != rot_dims // 2 or table.shape[2] != 2:
+                self._refuse(f"the rotation table must be [positions, {rot_dims // 2}, 2], got {tuple(table.shape)}")
+            positions = table.shape[0]
+            if ctx.max_seq_len > positions:
+                self._refuse("a request is longer than the rotation table")
+        self._step_arrays(ctx, tokens)
+        self._check(self._parts().akv_retention(
+            _ptr(projected), _long(projected.shape[1]), self._code_of(projected), ctx.num_seqs, heads, dim, vdim, rot_dims,
+            _ptr(table) if rot_dims else ctypes.c_void_p(0), positions, ctypes.c_float(key_scale), _ptr(decay),
+            ctypes.c_float(eps), _ptr(state), _long(state.shape[1]), _ptr(ctx.q_start), _ptr(ctx.seq_slots),
+            _ptr(ctx.positions), _ptr(out), self._stream()), "retention")
+
+    def gated_linear_scan(self, u, gates, gate_bias, rate, xy, blocks, state, taps, ctx, out) -> None:
+        """Per request and channel, token after token: a = exp(rate * sigmoid(gates_r + bias)), S <- a S + sqrt(1 - a^2)
+        sigmoid(gates_i + bias) u, out = S * gelu_tanh(y), with y the second half of `xy`'s columns and S at the start of
+        the request's state."""
+        tokens, channels = u.shape
+        self._dense(u, "u")
+        self._dense(gates, "gates", torch.float32, (tokens, blocks, 2 * (channels // blocks)))
+        self._dense(gate_bias, "gate_bias", torch.float32, (blocks, 2 * (channels // blocks)))
+        self._dense(rate, "rate", torch.float32, (channels,))
+        self._dense(xy, "xy", u.dtype, (tokens, 2 * channels))
+        self._dense(out, "out", u.dtype, (tokens, channels))
+        self._scan_state(state, ctx, channels, 1, taps)
+        self._step_arrays(ctx, tokens)
+        y = xy[:, channels:]
+        self._check(self._parts().akv_gated_linear_scan(
+            _ptr(u), self._code_of(u), _ptr(gates), _ptr(gate_bias), _ptr(rate), ctypes.c_void_p(y.data_ptr()),
+            _long(2 * channels), ctx.num_seqs, channels, blocks, _ptr(state), _long(state.shape[1]), _ptr(ctx.q_start),
+            _ptr(ctx.seq_slots), _ptr(out), self._stream()), "gated_linear_scan")
