@@ -1,4 +1,4 @@
-"""Prefill and decode throughput of the Keranex design at sizes that resemble a real model's layers (random weights),
+"""Prefill and decode throughput of the Keranex design (and, `--workload tukevik`, of the Tukevik design) at sizes that resemble a real model's layers (random weights),
 beside the dense Qwen3 decoder at equal width, depth, heads and active feed-forward width - the closest model the
 engine has.  `python bench.py --workload keranex [--design-sizes s,m] [--layers L]` prints one JSON line per size:
 
@@ -43,6 +43,39 @@ def keranex_config(size: dict, layers: int) -> dict:
             out.append(dict(type="latent_attention", mixer=latent(), mlp=mlp))
     return dict(architecture="Keranex", vocab=size["vocab"], width=size["width"], norm=dict(eps=1e-5),
                 embedding=dict(bigram=dict(buckets=size["vocab"] - 1, mul_prev=127, mul_cur=17)), layers=out)
+
+
+# Tukevik at sizes of the same widths: the pattern [attention over chunks beside retention + dense feed-forward, recurrent
+# unit + routed feed-forward, recurrent unit + dense, attention beside retention + routed]; a token uses `top` experts and
+# the shared one, as wide together as the dense feed-forward.
+TUKEVIK_SIZES = {
+    "s": dict(width=2048, vocab=32768, heads=16, kv_heads=4, dim=128, vdim=128, chunk=1024, r_heads=4, r_dim=128, r_vdim=128,
+              recurrent=2048, blocks=16, conv=4, experts=16, top=2, ff=1024, shared=1024, dense=3072),
+    "m": dict(width=4096, vocab=65536, heads=32, kv_heads=8, dim=128, vdim=128, chunk=2048, r_heads=8, r_dim=128, r_vdim=128,
+              recurrent=4096, blocks=16, conv=4, experts=32, top=4, ff=1024, shared=1024, dense=5120),
+}
+
+
+def tukevik_config(size: dict, layers: int) -> dict:
+    parallel = dict(
+        left=dict(heads=size["heads"], kv_heads=size["kv_heads"], dim=size["dim"], vdim=size["vdim"], mask=dict(size=size["chunk"]),
+                  scale=size["dim"] ** -0.5, softcap=30.0), left_scale=0.8,
+        right=dict(heads=size["r_heads"], dim=size["r_dim"], vdim=size["r_vdim"], rot=dict(base=1e6, dims=size["r_dim"]),
+                   decay=[1.0 - 2.0 ** -(5 + h % 6) for h in range(size["r_heads"])]), right_scale=1.1)
+    recurrent = dict(width=size["recurrent"], blocks=size["blocks"], conv=size["conv"])
+    dense = dict(kind="dense", ff=size["dense"])
+    routed = dict(kind="moe", expert=dict(ff=size["ff"]), router=dict(experts=size["experts"], top=size["top"]),
+                  shared=dict(ff=size["shared"]))
+    pattern = [("parallel", parallel, dense), ("rglru", recurrent, routed), ("rglru", recurrent, dense), ("parallel", parallel, routed)]
+    return dict(architecture="Tukevik", vocab=size["vocab"], width=size["width"], norm=dict(eps=1e-6), residual_mult=0.5,
+                layers=[dict(type=kind, mixer=mixer, mlp=mlp) for kind, mixer, mlp in (pattern[i % 4] for i in range(layers))])
+
+
+def qwen3_beside_tukevik(size: dict, layers: int) -> dict:
+    return dict(architectures=["Qwen3ForCausalLM"], num_hidden_layers=layers, hidden_size=size["width"],
+                num_attention_heads=size["heads"], num_key_value_heads=size["kv_heads"], head_dim=size["dim"],
+                intermediate_size=size["dense"], vocab_size=size["vocab"], rope_theta=1000000.0,
+                rms_norm_eps=1e-6, tie_word_embeddings=True, hidden_act="silu")
 
 
 def qwen3_config(size: dict, layers: int) -> dict:
@@ -103,8 +136,21 @@ def measure(config, batch: int, context: int, steps: int, warmup: int, graphs: b
 
 
 def design_workload(sizes: str, layers: int | None, batch: int, context: int, steps: int, warmup: int,
-                    graphs: bool = True, only: str = "") -> int:
-    from .config import KeranexConfig, Qwen3Config
+                    graphs: bool = True, only: str = "", design: str = "keranex") -> int:
+    from .config import KeranexConfig, Qwen3Config, TukevikConfig
+    for name in [s for s in sizes.split(",") if s and design == "tukevik"]:
+        size = TUKEVIK_SIZES[name]
+        count = layers or 8
+        line = {"workload": "tukevik", "sizes": name, "layers": count, "batch": batch, "context": context,
+                "prefill_tokens": PREFILL_TOKENS, "dtype": "bf16", "data": "synthetic: random-init weights, random token ids",
+                "shape": size}
+        if only in ("", "tukevik"):
+            line["tukevik"] = measure(TukevikConfig.from_dict(tukevik_config(size, count)), batch, context, steps, warmup, graphs)
+        if only in ("", "qwen3"):
+            line["qwen3_equal_size"] = measure(Qwen3Config.from_dict(qwen3_beside_tukevik(size, count)), batch, context, steps, warmup, graphs)
+        print(json.dumps(line), flush=True)
+    if design == "tukevik":
+        return 0
     for name in [s for s in sizes.split(",") if s]:
         size = SIZES[name]
         count = layers or 8

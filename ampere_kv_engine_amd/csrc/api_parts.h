@@ -46,6 +46,14 @@ int akv_gated_attention_rows(const void* q, const void* k_pages, const void* v_p
                              int kv_heads, int dim, int vdim, int page_size, long num_pages, float scale, float softcap,
                              int chunk, int window, int sink, hipStream_t stream);
 
+// The same for rows first_row .. tokens - 1 of a bfloat16 step, on the matrix cores: keys and values 32, 64, 128 or 256
+// wide, pages of a multiple of 16 tokens (-2 otherwise); a request's rows follow each other in the order of their positions.
+int akv_gated_attention_tiles(const void* q, const void* k_pages, const void* v_pages, const void* gates, long gate_stride,
+                              int gate_at, const int* seq_of_token, const int* q_start, const int* positions,
+                              const int* block_table, const int* table_rows, int table_width, void* out, int first_row,
+                              int tokens, int q_heads, int kv_heads, int dim, int vdim, int page_size, long num_pages,
+                              float scale, float softcap, int chunk, int window, int sink, hipStream_t stream);
+
 // ---- mixers with a state of fixed size (recurrent_mixers.hip) ----------------------------------------------------------
 // projected [tokens, stride]: rows [q | k (heads x dim each) | v | g (heads x vdim each)].  q and k are rotated over their
 // first rot_dims dimensions (pairs i, i + rot_dims / 2; `table` [positions, rot_dims / 2, 2] holds cos and sin), k times
@@ -55,12 +63,20 @@ int akv_retention(const void* projected, long stride, int dtype, int seqs, int h
                   const float* table, int table_positions, float key_scale, const float* decay, float eps, float* state,
                   long state_stride, const int* q_start, const int* seq_slots, const int* positions, void* out,
                   hipStream_t stream);
+// The same with every request's tokens cut into chunks of `length` that are worked on side by side - sums of k v^T per
+// chunk, the states before the chunks one after the other, then every chunk's outputs: `sums` holds 2 * seqs * heads *
+// chunks * dim * vdim floats, chunks = the most chunks a request of the step has.
+int akv_retention_chunked(const void* projected, long stride, int dtype, int seqs, int heads, int dim, int vdim, int rot_dims,
+                          const float* table, int table_positions, float key_scale, const float* decay, float eps,
+                          float* state, long state_stride, const int* q_start, const int* seq_slots, const int* positions,
+                          void* out, float* sums, int length, int chunks, hipStream_t stream);
 // u [tokens, channels]; gates [tokens, blocks, 2 * channels / blocks] float32 (a block's recurrence-gate logits, then its
 // input-gate logits) before their biases `gate_bias` [blocks, 2 * channels / blocks]; a = exp(rate[c] * sigmoid(.));
 // S [channels] at the start of a slot's state <- a S + sqrt(1 - a^2) sigmoid(.) u; out = S * gelu_tanh(y), y at
-// `y_stride` per token.
+// `y_stride` per token.  A request's tokens are cut into `runs` runs (1 .. 16), a wave each, whose decays' products and sums
+// are folded in the order of the runs.
 int akv_gated_linear_scan(const void* u, int dtype, const float* gates, const float* gate_bias, const float* rate,
-                          const void* y, long y_stride, int seqs, int channels, int blocks, float* state,
+                          const void* y, long y_stride, int seqs, int channels, int blocks, int runs, float* state,
                           long state_stride, const int* q_start, const int* seq_slots, void* out, hipStream_t stream);
 
 // ---- attention over a compressed latent (latent_attention.hip) ------------------------------------------------------

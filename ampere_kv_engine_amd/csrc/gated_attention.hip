@@ -147,9 +147,180 @@ __global__ __launch_bounds__(256) void gated_attention_rows_kernel(
   }
 }
 
+// ---- prompt portions on the matrix cores ----------------------------------------------------------------------------
+// bfloat16, keys 16 DT and values 16 VT wide, pages of a multiple of 16 tokens.  A wave is 16 neighbouring rows of the
+// step and one query head.  S^T = K Q^T (16 keys x 16 queries a step, the keys as A operand straight from the page) leaves
+// lane (c = l % 16, g = l / 16) with the scores of keys 4 g .. 4 g + 3 for query c - which is where the B operand of
+// O^T = V^T P^T wants the weights, so they never leave the registers; the values, [vdim, page] in the page, are its A
+// operand as they lie.  Scores, softcap, maxima, weights and sums are float32; a weight enters the second product as
+// two bfloat16 (its rounding and what the rounding left).  Rows of one tile may belong to several requests (the end of
+// one portion and the start of the next): the wave then takes the requests one after the other, each over its own keys,
+// with the other requests' columns switched off.  Key tiles lie at absolute positions.
+typedef __attribute__((ext_vector_type(4))) short short4_t;
+typedef __attribute__((ext_vector_type(4))) float float4_t;
+
+__device__ __forceinline__ short4_t load_bf16x4(const bf16_t* p) {
+  return __builtin_bit_cast(short4_t, *reinterpret_cast<const uint2*>(p));
+}
+
+template <int DT, int VT>
+__global__ __launch_bounds__(256) void gated_attention_tiles_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
+    const bf16_t* __restrict__ gates, long gate_stride, int gate_at, const int* __restrict__ seq_of_token,
+    const int* __restrict__ q_start, const int* __restrict__ positions, const int* __restrict__ block_table,
+    const int* __restrict__ table_rows, int table_width, bf16_t* __restrict__ out, int first_row, int tokens, int q_heads,
+    int kv_heads, int page_size, long num_pages, float scale, float softcap, int chunk, int window, int sink) {
+  constexpr int DIM = 16 * DT, VDIM = 16 * VT;
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
+  const int tiles = (tokens - first_row + 15) / 16;
+  const long item = static_cast<long>(blockIdx.x) * (blockDim.x / kWave) + wave;
+  if (item >= static_cast<long>(tiles) * q_heads) return;
+  const int head = static_cast<int>(item % q_heads), tile = static_cast<int>(item / q_heads);
+  const int kvh = head / (q_heads / kv_heads);
+  const int col = lane & 15, grp = lane >> 4;
+  const int row0 = first_row + tile * 16, row_end = min(row0 + 16, tokens);
+  const int my_row = row0 + col;
+  const bool have = my_row < row_end;
+  int my_pos = -1, my_lowest = 0;
+  short4_t qb[DT];
+  if (have) {
+    my_pos = positions[my_row];
+    my_lowest = window > 0 ? max(0, my_pos - window + 1) : 0;
+    if (chunk > 0) my_lowest = max(my_lowest, my_pos / chunk * chunk);
+    const bf16_t* qp = q + (static_cast<long>(my_row) * q_heads + head) * DIM + grp * 4;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) qb[dt] = load_bf16x4(qp + dt * 16);
+  } else {
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) qb[dt] = short4_t{0, 0, 0, 0};
+  }
+  float m = sink ? 0.f : -INFINITY, l = sink ? 1.f : 0.f;
+  float4_t o[VT];
+#pragma unroll
+  for (int vt = 0; vt < VT; ++vt) o[vt] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+  int row = row0;
+  while (row < row_end) {
+    const int r = seq_of_token[row];
+    const int run_end = min(row_end, q_start[r + 1]);
+    const int p_first = positions[row], p_last = p_first + (run_end - row - 1);
+    int lo_run = window > 0 ? max(0, p_first - window + 1) : 0;
+    if (chunk > 0) lo_run = max(lo_run, p_first / chunk * chunk);
+    const long table_at = static_cast<long>(table_rows != nullptr ? table_rows[r] : r) * table_width;
+    const bool in_run = have && my_row >= row && my_row < run_end;
+    for (int j0 = lo_run & ~15; j0 <= p_last; j0 += 16) {
+      const long page = block_table[table_at + j0 / page_size];
+      if (page < 0 || page >= num_pages) continue;      // (uniform; a page that is not the request's is never read)
+      const int o0 = j0 % page_size;
+      const bf16_t* kp = k_pages + ((page * kv_heads + kvh) * page_size + o0 + col) * DIM + grp * 4;
+      float4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+        acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(load_bf16x4(kp + dt * 16), qb[dt], acc, 0, 0, 0);
+      float s[4];
+      float highest = -INFINITY;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int j = j0 + grp * 4 + i;
+        float v = acc[i] * scale;
+        if (softcap > 0.f) v = softcap * tanhf(v / softcap);
+        s[i] = (in_run && j >= my_lowest && j <= my_pos) ? v : -INFINITY;
+        highest = fmaxf(highest, s[i]);
+      }
+      highest = fmaxf(highest, __shfl_xor(highest, 16, kWave));
+      highest = fmaxf(highest, __shfl_xor(highest, 32, kWave));
+      const float m_new = fmaxf(m, highest);
+      const float correction = m_new == m ? 1.f : expf(m - m_new);
+      float p[4], added = 0.f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        p[i] = s[i] == -INFINITY ? 0.f : expf(s[i] - m_new);
+        added += p[i];
+      }
+      added += __shfl_xor(added, 16, kWave);
+      added += __shfl_xor(added, 32, kWave);
+      l = l * correction + added;
+      m = m_new;
+      short4_t p_high, p_low;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint16_t high = bf16_bits(p[i]);
+        p_high[i] = static_cast<short>(high);
+        p_low[i] = static_cast<short>(bf16_bits(p[i] - __uint_as_float(static_cast<uint32_t>(high) << 16)));
+      }
+      const bf16_t* vp = v_pages + ((page * kv_heads + kvh) * VDIM + col) * page_size + o0 + grp * 4;
+      const int beyond = j0 + grp * 4 + 3 - p_last;      // this many of the lane's four keys are not written yet
+#pragma unroll
+      for (int vt = 0; vt < VT; ++vt) {
+        short4_t values = load_bf16x4(vp + static_cast<long>(vt) * 16 * page_size);
+        if (beyond > 0) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (i > 3 - beyond) values[i] = 0;
+        }
+        float4_t sum = o[vt];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) sum[i] *= correction;
+        sum = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(values, p_high, sum, 0, 0, 0);
+        o[vt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(values, p_low, sum, 0, 0, 0);
+      }
+    }
+    row = run_end;
+  }
+  if (!have) return;
+  float gate = 1.f;
+  if (gates != nullptr) gate = 1.f / (1.f + expf(-to_float(gates[static_cast<long>(my_row) * gate_stride + gate_at + head])));
+  const float factor = gate / l;
+  bf16_t* dst = out + (static_cast<long>(my_row) * q_heads + head) * VDIM + grp * 4;
+#pragma unroll
+  for (int vt = 0; vt < VT; ++vt) {
+    uint2 packed;
+    packed.x = bf16_pair(o[vt][0] * factor, o[vt][1] * factor);
+    packed.y = bf16_pair(o[vt][2] * factor, o[vt][3] * factor);
+    *reinterpret_cast<uint2*>(dst + vt * 16) = packed;
+  }
+}
+
 }  // namespace
 
 extern "C" {
+
+// The same for rows first_row .. tokens - 1 of a bfloat16 step on the matrix cores: keys and values of 32, 64, 128 or 256,
+// pages of a multiple of 16 tokens (-2 otherwise).  Rows of a request follow each other in the order of their positions.
+int akv_gated_attention_tiles(const void* q, const void* k_pages, const void* v_pages, const void* gates, long gate_stride,
+                              int gate_at, const int* seq_of_token, const int* q_start, const int* positions,
+                              const int* block_table, const int* table_rows, int table_width, void* out, int first_row,
+                              int tokens, int q_heads, int kv_heads, int dim, int vdim, int page_size, long num_pages,
+                              float scale, float softcap, int chunk, int window, int sink, hipStream_t stream) {
+  if (tokens <= first_row) return 0;
+  if (page_size % 16 != 0 || q_heads % kv_heads != 0) return -2;
+  const long items = static_cast<long>((tokens - first_row + 15) / 16) * q_heads;
+  const unsigned grid = static_cast<unsigned>((items + 3) / 4);
+#define AKV_TILES(DT, VT)                                                                                              \
+  gated_attention_tiles_kernel<DT, VT><<<grid, 256, 0, stream>>>(                                                      \
+      static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_pages), static_cast<const bf16_t*>(v_pages),         \
+      static_cast<const bf16_t*>(gates), gate_stride, gate_at, seq_of_token, q_start, positions, block_table, table_rows, \
+      table_width, static_cast<bf16_t*>(out), first_row, tokens, q_heads, kv_heads, page_size, num_pages, scale, softcap, \
+      chunk, window, sink)
+#define AKV_TILES_V(DT)                    \
+  switch (vdim) {                          \
+    case 32: AKV_TILES(DT, 2); break;      \
+    case 64: AKV_TILES(DT, 4); break;      \
+    case 128: AKV_TILES(DT, 8); break;     \
+    case 256: AKV_TILES(DT, 16); break;    \
+    default: return -2;                    \
+  }
+  switch (dim) {
+    case 32: AKV_TILES_V(2); break;
+    case 64: AKV_TILES_V(4); break;
+    case 128: AKV_TILES_V(8); break;
+    case 256: AKV_TILES_V(16); break;
+    default: return -2;
+  }
+#undef AKV_TILES_V
+#undef AKV_TILES
+  return AKV_LAUNCH_STATUS();
+}
 
 int akv_unit_norm_write(const void* projected, long stride, int dtype, long tokens, int q_heads, int kv_heads, int dim,
                         int vdim, float eps, int normed, const int* slot_map, void* k_pages, void* v_pages, int page_size,

@@ -119,45 +119,220 @@ __global__ __launch_bounds__(1024) void retention_kernel(
   }
 }
 
-// ---- gated linear recurrence ------------------------------------------------------------------------------------------
-// A thread is a (request, channel).  Tokens eight at a time: everything that does not depend on the state - gates,
-// decays, the fed values, gelu of the gating branch - is formed for the eight first, then the eight steps of S <- a S + f.
+// ---- retention over portions: chunks of L tokens side by side -----------------------------------------------------------
+// With w = decay:  S after a chunk = w^n S before + U,  U = sum_j w^(n - 1 - j) k_j v_j^T  (n tokens in the chunk), and
+// o_t = w^(t + 1) S_before^T q_t + sum_(j <= t) w^(t - j) (q_t . k_j) v_j.  Three launches: every chunk's U; per request and
+// head the states before its chunks, one after the other (U is replaced by them), and the request's new state; every
+// chunk's outputs, normed and gated.  All of float32.
+__device__ __forceinline__ float power(float w, int n) { return n == 0 ? 1.f : powf(w, static_cast<float>(n)); }
+
+// rotated q (if `with_q`) and scaled rotated k of a chunk's tokens into LDS rows of `pitch` floats, its values into vs
 template <typename T>
-__global__ __launch_bounds__(256) void gated_linear_scan_kernel(
+__device__ __forceinline__ void load_chunk(const T* __restrict__ projected, long stride, int heads, int h, int dim, int vdim,
+                                           int rot_dims, const float* __restrict__ table, int table_positions,
+                                           float key_scale, const int* __restrict__ positions, int first, int n,
+                                           float* qs, float* ks, float* vs, int pitch, bool with_q) {
+  const long q_at = static_cast<long>(h) * dim, k_at = static_cast<long>(heads) * dim + q_at;
+  const long v_at = 2L * heads * dim + static_cast<long>(h) * vdim;
+  const int half = rot_dims / 2;
+  for (int index = threadIdx.x; index < n * dim; index += blockDim.x) {
+    const int t = index / dim, d = index % dim;
+    const T* row = projected + static_cast<long>(first + t) * stride;
+    float qv = with_q ? to_float(row[q_at + d]) : 0.f, kv = to_float(row[k_at + d]);
+    if (d < rot_dims) {
+      const int i = d < half ? d : d - half;
+      const int pos = min(positions[first + t], table_positions - 1);
+      const float c = table[(static_cast<long>(pos) * half + i) * 2], sn = table[(static_cast<long>(pos) * half + i) * 2 + 1];
+      const int other = d < half ? d + half : d - half;
+      const float ko = to_float(row[k_at + other]);
+      kv = d < half ? kv * c - ko * sn : kv * c + ko * sn;
+      if (with_q) {
+        const float qo = to_float(row[q_at + other]);
+        qv = d < half ? qv * c - qo * sn : qv * c + qo * sn;
+      }
+    }
+    if (with_q) qs[t * pitch + d] = qv;
+    ks[t * pitch + d] = kv * key_scale;
+  }
+  for (int index = threadIdx.x; index < n * vdim; index += blockDim.x)
+    vs[index] = to_float(projected[static_cast<long>(first + index / vdim) * stride + v_at + index % vdim]);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void retention_chunk_sums_kernel(
+    const T* __restrict__ projected, long stride, int heads, int dim, int vdim, int rot_dims,
+    const float* __restrict__ table, int table_positions, float key_scale, const float* __restrict__ decay,
+    const int* __restrict__ q_start, const int* __restrict__ positions, float* __restrict__ sums, int length, int chunks) {
+  extern __shared__ float lds[];
+  const int seq = blockIdx.x, h = blockIdx.y, chunk = blockIdx.z;
+  const int first = q_start[seq], count = q_start[seq + 1] - first;
+  if (chunk * length >= count) return;
+  const int n = min(length, count - chunk * length), pitch = dim + 1;
+  float* ks = lds;                   // [length][pitch]
+  float* vs = ks + length * pitch;   // [length][vdim]
+  float* ws = vs + length * vdim;    // [length]
+  load_chunk(projected, stride, heads, h, dim, vdim, rot_dims, table, table_positions, key_scale, positions,
+             first + chunk * length, n, nullptr, ks, vs, pitch, false);
+  const float w = decay[h];
+  for (int j = threadIdx.x; j < n; j += blockDim.x) ws[j] = power(w, n - 1 - j);
+  __syncthreads();
+  float* mine = sums + ((static_cast<long>(seq) * heads + h) * chunks + chunk) * dim * vdim;
+  for (int item = threadIdx.x; item < dim * vdim; item += blockDim.x) {
+    const int d = item / vdim, v = item % vdim;
+    float total = 0.f;
+    for (int j = 0; j < n; ++j) total = fmaf(ws[j] * ks[j * pitch + d], vs[j * vdim + v], total);
+    mine[item] = total;
+  }
+}
+
+// sums [seq][head][chunk][dim * vdim]: U of every chunk; before: the state before every chunk, laid out the same way
+__global__ __launch_bounds__(256) void retention_chunk_states_kernel(const float* __restrict__ sums,
+                                                                     float* __restrict__ before, float* __restrict__ state,
+                                                                     long state_stride, const float* __restrict__ decay,
+                                                                     const int* __restrict__ q_start,
+                                                                     const int* __restrict__ seq_slots, int heads,
+                                                                     int size, int length, int chunks) {
+  const int seq = blockIdx.x, h = blockIdx.y;
+  const int item = blockIdx.z * blockDim.x + threadIdx.x;
+  if (item >= size) return;
+  const int count = q_start[seq + 1] - q_start[seq];
+  float* kept = state + static_cast<long>(seq_slots[seq]) * state_stride + static_cast<long>(h) * size + item;
+  const long base = (static_cast<long>(seq) * heads + h) * chunks * size + item;
+  const float w = decay[h], whole = power(w, length);
+  float S = *kept;
+#pragma unroll 8
+  for (int chunk = 0; chunk * length < count; ++chunk) {
+    const int n = min(length, count - chunk * length);
+    const float added = sums[base + static_cast<long>(chunk) * size];
+    before[base + static_cast<long>(chunk) * size] = S;
+    S = fmaf(n == length ? whole : power(w, n), S, added);
+  }
+  *kept = S;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void retention_chunk_outputs_kernel(
+    const T* __restrict__ projected, long stride, int heads, int dim, int vdim, int rot_dims,
+    const float* __restrict__ table, int table_positions, float key_scale, const float* __restrict__ decay, float eps,
+    const int* __restrict__ q_start, const int* __restrict__ positions, const float* __restrict__ states, int length,
+    int chunks, T* __restrict__ out) {
+  extern __shared__ float lds[];
+  const int seq = blockIdx.x, h = blockIdx.y, chunk = blockIdx.z;
+  const int first = q_start[seq], count = q_start[seq + 1] - first;
+  if (chunk * length >= count) return;
+  const int n = min(length, count - chunk * length), pitch = dim + 1;
+  float* qs = lds;                   // [length][pitch]
+  float* ks = qs + length * pitch;   // [length][pitch]
+  float* vs = ks + length * pitch;   // [length][vdim]
+  float* os = vs + length * vdim;    // [length][vdim]
+  float* as = os + length * vdim;    // [length][length + 1]: w^(t - j) (q_t . k_j), j <= t
+  float* ws = as + length * (length + 1);   // [length + 1]: w^0 .. w^length
+  const int row0 = first + chunk * length;
+  load_chunk(projected, stride, heads, h, dim, vdim, rot_dims, table, table_positions, key_scale, positions, row0, n, qs, ks,
+             vs, pitch, true);
+  const float w = decay[h];
+  for (int j = threadIdx.x; j <= n; j += blockDim.x) ws[j] = power(w, j);
+  __syncthreads();
+  for (int item = threadIdx.x; item < n * n; item += blockDim.x) {
+    const int t = item / n, j = item % n;
+    float dot = 0.f;
+    if (j <= t) {
+      for (int d = 0; d < dim; ++d) dot = fmaf(qs[t * pitch + d], ks[j * pitch + d], dot);
+      dot *= ws[t - j];
+    }
+    as[t * (length + 1) + j] = dot;
+  }
+  __syncthreads();
+  const float* before = states + ((static_cast<long>(seq) * heads + h) * chunks + chunk) * dim * vdim;
+  for (int item = threadIdx.x; item < n * vdim; item += blockDim.x) {
+    const int t = item / vdim, v = item % vdim;
+    float carried = 0.f, within = 0.f;
+    for (int d = 0; d < dim; ++d) carried = fmaf(qs[t * pitch + d], before[static_cast<long>(d) * vdim + v], carried);
+    for (int j = 0; j <= t; ++j) within = fmaf(as[t * (length + 1) + j], vs[j * vdim + v], within);
+    os[item] = fmaf(ws[t + 1], carried, within);
+  }
+  __syncthreads();
+  const int waves = blockDim.x / kWave, wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
+  const long g_at = 2L * heads * dim + static_cast<long>(heads) * vdim + static_cast<long>(h) * vdim;
+  for (int t = wave; t < n; t += waves) {
+    float squares = 0.f;
+    for (int c = lane; c < vdim; c += kWave) squares += os[t * vdim + c] * os[t * vdim + c];
+    const float scale = rsqrtf(wave_sum(squares) / static_cast<float>(vdim) + eps);
+    const long row = row0 + t;
+    for (int c = lane; c < vdim; c += kWave) {
+      const float g = to_float(projected[row * stride + g_at + c]);
+      out[row * heads * vdim + static_cast<long>(h) * vdim + c] = from_float<T>(os[t * vdim + c] * scale * silu(g));
+    }
+  }
+}
+
+// ---- gated linear recurrence ------------------------------------------------------------------------------------------
+// A block is a request and 64 neighbouring channels; its waves cut the request's tokens of this step into as many runs.
+// Thread (run, channel) first takes its run from a state of zero - which gives the run's product of decays and what the
+// run adds -, the runs' pairs meet in LDS, every thread folds the pairs of the runs before its own onto the request's
+// state, and takes its run again from there, now writing S * gelu_tanh(y).  Tokens eight at a time: everything that
+// does not depend on the state - gates, decays, the fed values - is formed for the eight first.
+template <typename T>
+__global__ __launch_bounds__(1024) void gated_linear_scan_kernel(
     const T* __restrict__ u, const float* __restrict__ gates, const float* __restrict__ gate_bias,
     const float* __restrict__ rate, const T* __restrict__ y, long y_stride, int channels, int block_width,
     float* __restrict__ state, long state_stride, const int* __restrict__ q_start, const int* __restrict__ seq_slots,
     T* __restrict__ out) {
+  __shared__ float products[16][kWave], sums[16][kWave];
   const int seq = blockIdx.x;
-  const int c = blockIdx.y * blockDim.x + threadIdx.x;
-  if (c >= channels) return;
+  const int lane = threadIdx.x & (kWave - 1), run = threadIdx.x / kWave, runs = blockDim.x / kWave;
+  const int c = blockIdx.y * kWave + lane;
+  const bool live = c < channels;
   const int first = q_start[seq], count = q_start[seq + 1] - first;
-  const int b = c / block_width, j = c % block_width;
+  const int per_run = (count + runs - 1) / runs;
+  const int lo = min(run * per_run, count), hi = min(lo + per_run, count);
+  const int cc = live ? c : 0;
+  const int b = cc / block_width, j = cc % block_width;
   const long gate_at = static_cast<long>(b) * 2 * block_width + j;      // (recurrence gate; the input gate block_width on)
-  const float bias_r = gate_bias[gate_at], bias_i = gate_bias[gate_at + block_width], slope = rate[c];
-  float* mine = state + static_cast<long>(seq_slots[seq]) * state_stride + c;
-  float S = *mine;
+  const float bias_r = gate_bias[gate_at], bias_i = gate_bias[gate_at + block_width], slope = rate[cc];
+  float* mine = state + static_cast<long>(seq_slots[seq]) * state_stride + cc;
   constexpr int kStep = 8;
-  for (int base = 0; base < count; base += kStep) {
-    float a[kStep], f[kStep], gy[kStep];
+  float S = runs > 1 ? 0.f : *mine;
+  for (int pass = (runs > 1 ? 0 : 1); pass < 2; ++pass) {
+    float product = 1.f;
+    for (int base = lo; base < hi; base += kStep) {
+      float a[kStep], f[kStep];
 #pragma unroll
-    for (int t = 0; t < kStep; ++t) {
-      const long n = first + min(base + t, count - 1);
-      const float r = sigmoid(gates[n * 2 * channels + gate_at] + bias_r);
-      const float i = sigmoid(gates[n * 2 * channels + gate_at + block_width] + bias_i);
-      a[t] = expf(slope * r);
-      f[t] = sqrtf(1.f - a[t] * a[t]) * i * to_float(u[n * channels + c]);
-      gy[t] = gelu_tanh(to_float(y[n * y_stride + c]));
-    }
+      for (int t = 0; t < kStep; ++t) {
+        const long n = first + min(base + t, hi - 1);
+        const float r = sigmoid(gates[n * 2 * channels + gate_at] + bias_r);
+        const float i = sigmoid(gates[n * 2 * channels + gate_at + block_width] + bias_i);
+        a[t] = expf(slope * r);
+        f[t] = sqrtf(1.f - a[t] * a[t]) * i * to_float(u[n * channels + cc]);
+      }
+      if (pass == 0) {
 #pragma unroll
-    for (int t = 0; t < kStep; ++t) {
-      if (base + t < count) {
-        S = fmaf(a[t], S, f[t]);
-        out[static_cast<long>(first + base + t) * channels + c] = from_float<T>(S * gy[t]);
+        for (int t = 0; t < kStep; ++t) {
+          if (base + t < hi) {
+            S = fmaf(a[t], S, f[t]);
+            product *= a[t];
+          }
+        }
+      } else {
+#pragma unroll
+        for (int t = 0; t < kStep; ++t) {
+          if (base + t < hi) {
+            S = fmaf(a[t], S, f[t]);
+            const long n = first + base + t;
+            if (live) out[n * channels + c] = from_float<T>(S * gelu_tanh(to_float(y[n * y_stride + c])));
+          }
+        }
       }
     }
+    if (pass == 0) {
+      products[run][lane] = product;
+      sums[run][lane] = S;
+      __syncthreads();
+      S = *mine;
+      for (int before = 0; before < run; ++before) S = fmaf(products[before][lane], S, sums[before][lane]);
+    }
   }
-  *mine = S;
+  if (run == runs - 1 && live) *mine = S;
 }
 
 }  // namespace
@@ -202,13 +377,50 @@ int akv_retention(const void* projected, long stride, int dtype, int seqs, int h
   return AKV_LAUNCH_STATUS();
 }
 
+// The same over chunks of `length` tokens side by side (see above): `sums` holds 2 * seqs * heads * chunks * dim * vdim
+// floats (the chunks' sums, then the states before them), chunks = the most chunks a request of the step has.
+int akv_retention_chunked(const void* projected, long stride, int dtype, int seqs, int heads, int dim, int vdim, int rot_dims,
+                          const float* table, int table_positions, float key_scale, const float* decay, float eps,
+                          float* state, long state_stride, const int* q_start, const int* seq_slots, const int* positions,
+                          void* out, float* sums, int length, int chunks, hipStream_t stream) {
+  if (seqs <= 0 || chunks <= 0) return 0;
+  if (heads <= 0 || dim <= 0 || vdim <= 0 || rot_dims < 0 || rot_dims % 2 || rot_dims > dim || length < 1) return -2;
+  if (rot_dims > 0 && (table == nullptr || table_positions <= 0)) return -2;
+  const int pitch = dim + 1;
+  const size_t lds_sums = static_cast<size_t>(length * pitch + length * vdim + length) * 4;
+  const size_t lds_outputs = static_cast<size_t>(2 * length * pitch + 2 * length * vdim + length * (length + 1) + length + 1) * 4;
+  if (lds_sums > 128 * 1024 || lds_outputs > 128 * 1024) return -2;
+  const dim3 grid(seqs, heads, chunks);
+  const int size = dim * vdim;
+  float* states = sums + static_cast<long>(seqs) * heads * chunks * size;
+  AKV_DISPATCH(dtype, T, {
+    if (lds_sums > 64 * 1024 &&
+        hipFuncSetAttribute(reinterpret_cast<const void*>(&retention_chunk_sums_kernel<T>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_sums)) != hipSuccess)
+      return -2;
+    if (lds_outputs > 64 * 1024 &&
+        hipFuncSetAttribute(reinterpret_cast<const void*>(&retention_chunk_outputs_kernel<T>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_outputs)) != hipSuccess)
+      return -2;
+    retention_chunk_sums_kernel<T><<<grid, 256, lds_sums, stream>>>(static_cast<const T*>(projected), stride, heads, dim, vdim,
+                                                                  rot_dims, table, table_positions, key_scale, decay, q_start,
+                                                                  positions, sums, length, chunks);
+    retention_chunk_states_kernel<<<dim3(seqs, heads, (size + 255) / 256), 256, 0, stream>>>(
+        sums, states, state, state_stride, decay, q_start, seq_slots, heads, size, length, chunks);
+    retention_chunk_outputs_kernel<T><<<grid, 256, lds_outputs, stream>>>(
+        static_cast<const T*>(projected), stride, heads, dim, vdim, rot_dims, table, table_positions, key_scale, decay, eps,
+        q_start, positions, states, length, chunks, static_cast<T*>(out));
+  });
+  return AKV_LAUNCH_STATUS();
+}
+
 int akv_gated_linear_scan(const void* u, int dtype, const float* gates, const float* gate_bias, const float* rate,
-                          const void* y, long y_stride, int seqs, int channels, int blocks, float* state,
+                          const void* y, long y_stride, int seqs, int channels, int blocks, int runs, float* state,
                           long state_stride, const int* q_start, const int* seq_slots, void* out, hipStream_t stream) {
   if (seqs <= 0) return 0;
-  if (channels <= 0 || blocks <= 0 || channels % blocks) return -2;
-  const dim3 grid(seqs, (channels + 255) / 256);
-  AKV_DISPATCH(dtype, T, gated_linear_scan_kernel<T><<<grid, 256, 0, stream>>>(
+  if (channels <= 0 || blocks <= 0 || channels % blocks || runs < 1 || runs > 16) return -2;
+  const dim3 grid(seqs, (channels + kWave - 1) / kWave);
+  AKV_DISPATCH(dtype, T, gated_linear_scan_kernel<T><<<grid, runs * kWave, 0, stream>>>(
                              static_cast<const T*>(u), gates, gate_bias, rate, static_cast<const T*>(y), y_stride, channels,
                              channels / blocks, state, state_stride, q_start, seq_slots, static_cast<T*>(out)));
   return AKV_LAUNCH_STATUS();

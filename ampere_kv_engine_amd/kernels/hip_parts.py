@@ -40,7 +40,7 @@ class PartsKernels:
                          "akv_rotate_queries", "akv_heads_linear", "akv_latent_attend", "akv_latent_attend_mfma", "akv_conv_silu",
                          "akv_conv_state_update", "akv_selective_scan", "akv_route", "akv_gate_relu_squared",
                          "akv_parts_slot_layout", "akv_conv_taps", "akv_scaled_sum", "akv_unit_norm_write",
-                         "akv_gated_attention_rows", "akv_retention", "akv_gated_linear_scan", "akv_route_chosen",
+                         "akv_gated_attention_rows", "akv_gated_attention_tiles", "akv_retention", "akv_retention_chunked", "akv_gated_linear_scan", "akv_route_chosen",
                          "akv_gate_silu_mul"):
                 getattr(lib, name).restype = ctypes.c_int
             layout = (ctypes.c_int * 3)()
@@ -389,6 +389,7 @@ class PartsKernels:
 
     # ---- attention with unit-normed queries and keys, a softcap, chunks, a sink and a gate per head ----------------------
     MAX_VALUE_DIM = 256
+    MATRIX_CORE_HEAD_DIMS = (32, 64, 128, 256)      # widths of keys and of values that the portions' kernel is built for
 
     def check_gated_attention_sizes(self, q_heads: int, kv_heads: int, dim: int, vdim: int, page_size: int) -> None:
         if q_heads % kv_heads:
@@ -446,12 +447,24 @@ class PartsKernels:
             self._refuse("the block table has fewer rows than the step has requests")
         if ctx.max_seq_len > meta.width * page_size:
             self._refuse("a request is longer than its row of the block table")
-        self._check(self._parts().akv_gated_attention_rows(
-            _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(gates), _long(gate_stride), gate_at, _ptr(ctx.seq_of_token),
-            _ptr(ctx.positions), _ptr(meta.block_table), _ptr(meta.rows), meta.width, _ptr(out), self._code_of(q),
-            _long(tokens), q_heads, kv_heads, dim, vdim, page_size, _long(num_pages), ctypes.c_float(scale),
-            ctypes.c_float(softcap if softcap is not None else 0.0), int(chunk) if chunk is not None else 0,
-            int(window) if window is not None else 0, 1 if sink else 0, self._stream()), "gated_attention")
+        tail = (ctypes.c_float(scale), ctypes.c_float(softcap if softcap is not None else 0.0),
+                int(chunk) if chunk is not None else 0, int(window) if window is not None else 0, 1 if sink else 0,
+                self._stream())
+        singles = tokens
+        if (q.dtype == torch.bfloat16 and dim in self.MATRIX_CORE_HEAD_DIMS and vdim in self.MATRIX_CORE_HEAD_DIMS
+                and page_size % 16 == 0):
+            # single tokens: a wave per token and head; the portions' rows, which follow them, go to the matrix cores
+            singles = ctx.num_decode_seqs
+            self._check(self._parts().akv_gated_attention_tiles(
+                _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(gates), _long(gate_stride), gate_at, _ptr(ctx.seq_of_token),
+                _ptr(ctx.q_start), _ptr(ctx.positions), _ptr(meta.block_table), _ptr(meta.rows), meta.width, _ptr(out),
+                singles, tokens, q_heads, kv_heads, dim, vdim, page_size, _long(num_pages), *tail),
+                "gated_attention on the matrix cores")
+        if singles:
+            self._check(self._parts().akv_gated_attention_rows(
+                _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(gates), _long(gate_stride), gate_at, _ptr(ctx.seq_of_token),
+                _ptr(ctx.positions), _ptr(meta.block_table), _ptr(meta.rows), meta.width, _ptr(out), self._code_of(q),
+                _long(singles), q_heads, kv_heads, dim, vdim, page_size, _long(num_pages), *tail), "gated_attention")
 
     # ---- mixers with a state of fixed size -----------------------------------------------------------------------------
     def check_retention_sizes(self, heads: int, dim: int, vdim: int) -> None:
@@ -475,15 +488,47 @@ class PartsKernels:
             self._dense(table, "table", torch.float32)
             if table.dim() != 3 or table.shape[1] != rot_dims // 2 or table.shape[2] != 2:
                 self._refuse(f"the rotation table must be [positions, {rot_dims // 2}, 2], got {tuple(table.shape)}")
-            positions = table.shape[0]
-            if ctx.max_seq_len > positions:
-                self._refuse("a request is longer than the rotation table")
+            positions = table.shape[0]       # (the engine admits no request beyond the positions its tables were built for)
         self._step_arrays(ctx, tokens)
-        self._check(self._parts().akv_retention(
-            _ptr(projected), _long(projected.shape[1]), self._code_of(projected), ctx.num_seqs, heads, dim, vdim, rot_dims,
-            _ptr(table) if rot_dims else ctypes.c_void_p(0), positions, ctypes.c_float(key_scale), _ptr(decay),
-            ctypes.c_float(eps), _ptr(state), _long(state.shape[1]), _ptr(ctx.q_start), _ptr(ctx.seq_slots),
-            _ptr(ctx.positions), _ptr(out), self._stream()), "retention")
+        head = (_ptr(projected), _long(projected.shape[1]), self._code_of(projected), ctx.num_seqs, heads, dim, vdim, rot_dims,
+                _ptr(table) if rot_dims else ctypes.c_void_p(0), positions, ctypes.c_float(key_scale), _ptr(decay),
+                ctypes.c_float(eps), _ptr(state), _long(state.shape[1]), _ptr(ctx.q_start), _ptr(ctx.seq_slots),
+                _ptr(ctx.positions), _ptr(out))
+        length = self._retention_chunk(dim, vdim)
+        if ctx.max_new_tokens >= self.RETENTION_CHUNKED_FROM and length:
+            # portions: chunks side by side (the step's shape alone decides, so a recorded step replays the same launches)
+            chunks = (ctx.max_new_tokens + length - 1) // length
+            sums = self._retention_sums(2 * ctx.num_seqs * heads * chunks * dim * vdim)
+            self._check(self._parts().akv_retention_chunked(*head, _ptr(sums), length, chunks, self._stream()),
+                        "retention over chunks")
+            return
+        self._check(self._parts().akv_retention(*head, self._stream()), "retention")
+
+    RETENTION_CHUNKED_FROM = 24       # steps whose longest portion has fewer tokens take them one after the other
+
+    @staticmethod
+    def _retention_chunk(dim: int, vdim: int) -> int:
+        """Tokens per chunk: the most of 32, 16, 8 whose operands fit into 128 KB of LDS (0: none does)."""
+        for length in (32, 16, 8):
+            if (2 * length * (dim + 1) + 2 * length * vdim + length * (length + 1) + length + 1) * 4 <= 128 * 1024:
+                return length
+        return 0
+
+    def _retention_sums(self, need: int) -> torch.Tensor:
+        """Where the chunks' sums and the states before them lie during a step."""
+        held = self.__dict__.get("_retention_buffer")
+        if held is None or held.numel() < need:
+            if torch.cuda.is_current_stream_capturing():
+                self._refuse("a recorded step needs more room for retention's chunks than the steps before it")
+            self.__dict__.setdefault("_retention_outgrown", []).append(held)
+            held = self.__dict__["_retention_buffer"] = torch.empty(max(need, 1 << 22), dtype=torch.float32, device=self.device)
+        return held
+
+    @staticmethod
+    def _scan_runs(longest_portion: int) -> int:
+        """Runs that the longest portion of a step is cut into: about 32 tokens a run, 16 runs at most (the step's shape
+        alone decides, so a recorded step is cut as the same step run eagerly)."""
+        return max(1, min(16, longest_portion // 32))
 
     def gated_linear_scan(self, u, gates, gate_bias, rate, xy, blocks, state, taps, ctx, out) -> None:
         """Per request and channel, token after token: a = exp(rate * sigmoid(gates_r + bias)), S <- a S + sqrt(1 - a^2)
@@ -501,5 +546,6 @@ class PartsKernels:
         y = xy[:, channels:]
         self._check(self._parts().akv_gated_linear_scan(
             _ptr(u), self._code_of(u), _ptr(gates), _ptr(gate_bias), _ptr(rate), ctypes.c_void_p(y.data_ptr()),
-            _long(2 * channels), ctx.num_seqs, channels, blocks, _ptr(state), _long(state.shape[1]), _ptr(ctx.q_start),
+            _long(2 * channels), ctx.num_seqs, channels, blocks, self._scan_runs(ctx.max_new_tokens), _ptr(state),
+            _long(state.shape[1]), _ptr(ctx.q_start),
             _ptr(ctx.seq_slots), _ptr(out), self._stream()), "gated_linear_scan")

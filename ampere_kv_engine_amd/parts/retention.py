@@ -46,10 +46,10 @@ class Retention(Part):
             # the frequencies rounded once from double precision; cos and sin of every position the engine can reach,
             # float32 [max_seq_len, rotary_dims / 2, 2], one table for all layers with the same constants
             half = self.rot_dims // 2
+            reach = (runtime.max_seq_len + runtime.page_size - 1) // runtime.page_size * runtime.page_size     # whole pages
             freq = torch.from_numpy((self.base ** (-2.0 * np.arange(half, dtype=np.float64) / self.rot_dims)).astype(np.float32))
             self.table = runtime.shared_buffer(
-                ("rotary_first_dims", self.rot_dims, self.base, runtime.max_seq_len),
-                (runtime.max_seq_len, half, 2), torch.float32,
+                ("rotary_first_dims", self.rot_dims, self.base, reach), (reach, half, 2), torch.float32,
                 lambda table: runtime.kernels.rope_table(freq.to(runtime.device), table))
         runtime.kernels.check_retention_sizes(self.heads, self.dim, self.vdim)
 

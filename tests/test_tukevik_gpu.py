@@ -157,7 +157,8 @@ def _ctx(lengths_before, counts, device=DEVICE):
         seq_of_token += [r] * count
     ints = lambda values: torch.tensor(values, dtype=torch.int32, device=device)
     seqs = len(counts)
-    return SimpleNamespace(num_seqs=seqs, num_tokens=q_start[-1], q_start=ints(q_start), positions=ints(positions),
+    singles = next((r for r, count in enumerate(counts) if count != 1), seqs)        # single tokens come first in a step
+    return SimpleNamespace(num_decode_seqs=singles, max_new_tokens=max(counts), num_seqs=seqs, num_tokens=q_start[-1], q_start=ints(q_start), positions=ints(positions),
                            seq_of_token=ints(seq_of_token), seq_slots=ints(list(range(seqs))), host_q_start=q_start,
                            host_seq_slots=list(range(seqs)), host_seq_lens=[b + c for b, c in zip(lengths_before, counts)],
                            max_seq_len=max(b + c for b, c in zip(lengths_before, counts)))
@@ -165,7 +166,8 @@ def _ctx(lengths_before, counts, device=DEVICE):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("heads,kv_heads,dim,vdim,chunk,page", [(4, 2, 16, 24, 11, 4), (3, 1, 40, 8, 64, 16), (8, 8, 64, 64, 7, 8),
-                                                               (2, 1, 128, 256, 300, 16)])
+                                                               (2, 1, 128, 256, 300, 16), (8, 2, 64, 32, 20, 16),
+                                                               (4, 4, 32, 128, 48, 32)])
 def test_attention_kernel_alone(hip, dtype, heads, kv_heads, dim, vdim, chunk, page):
     """Two requests in two portions each, through the unit norm with its cache write and the attention, against the plain
     attention of the whole sequences.  Scores are made sharp, and one key a request - the first of a chunk - is made to
