@@ -39,12 +39,12 @@ int akv_unit_norm_write(const void* projected, long stride, int dtype, long toke
 // out [tokens, q_heads, vdim].  score = (q . k) * scale, then softcap * tanh(score / softcap) where softcap > 0; a query at
 // position p sees the keys j <= p with j > p - window (window > 0) and floor(j / chunk) = floor(p / chunk) (chunk > 0);
 // with `sink` the softmax's denominator has one more term exp(0); with `gates` head h's output is multiplied by
-// sigmoid(gates[t * gate_stride + gate_at + h]).
+// sigmoid(gates[t * gate_stride + gate_at + h]).  A token's outputs lie at out + t * out_stride, times out_scale.
 int akv_gated_attention_rows(const void* q, const void* k_pages, const void* v_pages, const void* gates, long gate_stride,
                              int gate_at, const int* seq_of_token, const int* positions, const int* block_table,
                              const int* table_rows, int table_width, void* out, int dtype, long tokens, int q_heads,
                              int kv_heads, int dim, int vdim, int page_size, long num_pages, float scale, float softcap,
-                             int chunk, int window, int sink, hipStream_t stream);
+                             int chunk, int window, int sink, long out_stride, float out_scale, hipStream_t stream);
 
 // The same for rows first_row .. tokens - 1 of a bfloat16 step, on the matrix cores: keys and values 32, 64, 128 or 256
 // wide, pages of a multiple of 16 tokens (-2 otherwise); a request's rows follow each other in the order of their positions.
@@ -52,28 +52,30 @@ int akv_gated_attention_tiles(const void* q, const void* k_pages, const void* v_
                               int gate_at, const int* seq_of_token, const int* q_start, const int* positions,
                               const int* block_table, const int* table_rows, int table_width, void* out, int first_row,
                               int tokens, int q_heads, int kv_heads, int dim, int vdim, int page_size, long num_pages,
-                              float scale, float softcap, int chunk, int window, int sink, hipStream_t stream);
+                              float scale, float softcap, int chunk, int window, int sink, long out_stride, float out_scale,
+                              hipStream_t stream);
 
 // ---- mixers with a state of fixed size (recurrent_mixers.hip) ----------------------------------------------------------
 // projected [tokens, stride]: rows [q | k (heads x dim each) | v | g (heads x vdim each)].  q and k are rotated over their
 // first rot_dims dimensions (pairs i, i + rot_dims / 2; `table` [positions, rot_dims / 2, 2] holds cos and sin), k times
 // key_scale; per request and head S [dim, vdim] (at state[slot * state_stride + head * dim * vdim]) <- decay S + k v^T,
-// o = S^T q; out [tokens, heads, vdim] = o / rms(o) * silu(g).
+// o = S^T q; out [tokens, heads, vdim] (a token's at out + t * out_stride) = o / rms(o) * silu(g) * out_scale.
 int akv_retention(const void* projected, long stride, int dtype, int seqs, int heads, int dim, int vdim, int rot_dims,
                   const float* table, int table_positions, float key_scale, const float* decay, float eps, float* state,
                   long state_stride, const int* q_start, const int* seq_slots, const int* positions, void* out,
-                  hipStream_t stream);
+                  long out_stride, float out_scale, hipStream_t stream);
 // The same with every request's tokens cut into chunks of `length` that are worked on side by side - sums of k v^T per
 // chunk, the states before the chunks one after the other, then every chunk's outputs: `sums` holds 2 * seqs * heads *
 // chunks * dim * vdim floats, chunks = the most chunks a request of the step has.
 int akv_retention_chunked(const void* projected, long stride, int dtype, int seqs, int heads, int dim, int vdim, int rot_dims,
                           const float* table, int table_positions, float key_scale, const float* decay, float eps,
                           float* state, long state_stride, const int* q_start, const int* seq_slots, const int* positions,
-                          void* out, float* sums, int length, int chunks, hipStream_t stream);
+                          void* out, long out_stride, float out_scale, float* sums, int length, int chunks,
+                          hipStream_t stream);
 // u [tokens, channels]; gates [tokens, blocks, 2 * channels / blocks] float32 (a block's recurrence-gate logits, then its
 // input-gate logits) before their biases `gate_bias` [blocks, 2 * channels / blocks]; a = exp(rate[c] * sigmoid(.));
 // S [channels] at the start of a slot's state <- a S + sqrt(1 - a^2) sigmoid(.) u; out = S * gelu_tanh(y), y at
-// `y_stride` per token.  A request's tokens are cut into `runs` runs (1 .. 16), a wave each, whose decays' products and sums
+// `y_stride` per token.  A request's tokens are cut into `runs` runs (1 .. 64) whose decays' products and sums
 // are folded in the order of the runs.
 int akv_gated_linear_scan(const void* u, int dtype, const float* gates, const float* gate_bias, const float* rate,
                           const void* y, long y_stride, int seqs, int channels, int blocks, int runs, float* state,

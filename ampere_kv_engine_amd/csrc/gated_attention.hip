@@ -75,7 +75,7 @@ __global__ __launch_bounds__(256) void gated_attention_rows_kernel(
     long gate_stride, int gate_at, const int* __restrict__ seq_of_token, const int* __restrict__ positions,
     const int* __restrict__ block_table, const int* __restrict__ table_rows, int table_width, T* __restrict__ out,
     long tokens, int q_heads, int kv_heads, int dim, int vdim, int page_size, long num_pages, float scale, float softcap,
-    int chunk, int window, int sink) {
+    int chunk, int window, int sink, long out_stride, float out_scale) {
   extern __shared__ unsigned char lds_raw[];
   const int waves = blockDim.x / kWave, wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
   const long row = static_cast<long>(blockIdx.x) * waves + wave;
@@ -138,12 +138,12 @@ __global__ __launch_bounds__(256) void gated_attention_rows_kernel(
     }
     wave_sync_lds();
   }
-  float gate = 1.f;
-  if (gates != nullptr) gate = 1.f / (1.f + expf(-to_float(gates[n * gate_stride + gate_at + h])));
+  float gate = out_scale;
+  if (gates != nullptr) gate = out_scale / (1.f + expf(-to_float(gates[n * gate_stride + gate_at + h])));
 #pragma unroll
   for (int c = 0; c < kMaxValueRegs; ++c) {
     const int i = lane + c * kWave;
-    if (i < vdim) out[row * vdim + i] = from_float<T>(acc[c] / l * gate);
+    if (i < vdim) out[n * out_stride + static_cast<long>(h) * vdim + i] = from_float<T>(acc[c] / l * gate);
   }
 }
 
@@ -163,14 +163,20 @@ __device__ __forceinline__ short4_t load_bf16x4(const bf16_t* p) {
   return __builtin_bit_cast(short4_t, *reinterpret_cast<const uint2*>(p));
 }
 
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+
+__device__ __forceinline__ uint4 load_bf16x8(const bf16_t* p) { return *reinterpret_cast<const uint4*>(p); }
+
+// DT: key width / 32 (the first product runs in steps of 32 dimensions), VT: value width / 16.
 template <int DT, int VT>
 __global__ __launch_bounds__(256) void gated_attention_tiles_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     const bf16_t* __restrict__ gates, long gate_stride, int gate_at, const int* __restrict__ seq_of_token,
     const int* __restrict__ q_start, const int* __restrict__ positions, const int* __restrict__ block_table,
     const int* __restrict__ table_rows, int table_width, bf16_t* __restrict__ out, int first_row, int tokens, int q_heads,
-    int kv_heads, int page_size, long num_pages, float scale, float softcap, int chunk, int window, int sink) {
-  constexpr int DIM = 16 * DT, VDIM = 16 * VT;
+    int kv_heads, int page_size, long num_pages, float scale, float softcap, int chunk, int window, int sink,
+    long out_stride, float out_scale) {
+  constexpr int DIM = 32 * DT, VDIM = 16 * VT;
   const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
   const int tiles = (tokens - first_row + 15) / 16;
   const long item = static_cast<long>(blockIdx.x) * (blockDim.x / kWave) + wave;
@@ -182,17 +188,17 @@ __global__ __launch_bounds__(256) void gated_attention_tiles_kernel(
   const int my_row = row0 + col;
   const bool have = my_row < row_end;
   int my_pos = -1, my_lowest = 0;
-  short4_t qb[DT];
+  uint4 qb[DT];
   if (have) {
     my_pos = positions[my_row];
     my_lowest = window > 0 ? max(0, my_pos - window + 1) : 0;
     if (chunk > 0) my_lowest = max(my_lowest, my_pos / chunk * chunk);
-    const bf16_t* qp = q + (static_cast<long>(my_row) * q_heads + head) * DIM + grp * 4;
+    const bf16_t* qp = q + (static_cast<long>(my_row) * q_heads + head) * DIM + grp * 8;
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) qb[dt] = load_bf16x4(qp + dt * 16);
+    for (int dt = 0; dt < DT; ++dt) qb[dt] = load_bf16x8(qp + dt * 32);
   } else {
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) qb[dt] = short4_t{0, 0, 0, 0};
+    for (int dt = 0; dt < DT; ++dt) qb[dt] = make_uint4(0u, 0u, 0u, 0u);
   }
   float m = sink ? 0.f : -INFINITY, l = sink ? 1.f : 0.f;
   float4_t o[VT];
@@ -208,70 +214,92 @@ __global__ __launch_bounds__(256) void gated_attention_tiles_kernel(
     if (chunk > 0) lo_run = max(lo_run, p_first / chunk * chunk);
     const long table_at = static_cast<long>(table_rows != nullptr ? table_rows[r] : r) * table_width;
     const bool in_run = have && my_row >= row && my_row < run_end;
-    for (int j0 = lo_run & ~15; j0 <= p_last; j0 += 16) {
+    // a step's keys and values are asked for while the step before is worked on
+    uint4 keys[DT], keys_next[DT];
+    short4_t values[VT], values_next[VT];
+    bool there = false, there_next = false;
+    auto fetch = [&](int j0, uint4 (&ks)[DT], short4_t (&vs)[VT]) -> bool {
       const long page = block_table[table_at + j0 / page_size];
-      if (page < 0 || page >= num_pages) continue;      // (uniform; a page that is not the request's is never read)
+      if (page < 0 || page >= num_pages) return false;      // (uniform; a page that is not the request's is never read)
       const int o0 = j0 % page_size;
-      const bf16_t* kp = k_pages + ((page * kv_heads + kvh) * page_size + o0 + col) * DIM + grp * 4;
-      float4_t acc = {0.f, 0.f, 0.f, 0.f};
+      const bf16_t* kp = k_pages + ((page * kv_heads + kvh) * page_size + o0 + col) * DIM + grp * 8;
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt)
-        acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(load_bf16x4(kp + dt * 16), qb[dt], acc, 0, 0, 0);
-      float s[4];
-      float highest = -INFINITY;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int j = j0 + grp * 4 + i;
-        float v = acc[i] * scale;
-        if (softcap > 0.f) v = softcap * tanhf(v / softcap);
-        s[i] = (in_run && j >= my_lowest && j <= my_pos) ? v : -INFINITY;
-        highest = fmaxf(highest, s[i]);
-      }
-      highest = fmaxf(highest, __shfl_xor(highest, 16, kWave));
-      highest = fmaxf(highest, __shfl_xor(highest, 32, kWave));
-      const float m_new = fmaxf(m, highest);
-      const float correction = m_new == m ? 1.f : expf(m - m_new);
-      float p[4], added = 0.f;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        p[i] = s[i] == -INFINITY ? 0.f : expf(s[i] - m_new);
-        added += p[i];
-      }
-      added += __shfl_xor(added, 16, kWave);
-      added += __shfl_xor(added, 32, kWave);
-      l = l * correction + added;
-      m = m_new;
-      short4_t p_high, p_low;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const uint16_t high = bf16_bits(p[i]);
-        p_high[i] = static_cast<short>(high);
-        p_low[i] = static_cast<short>(bf16_bits(p[i] - __uint_as_float(static_cast<uint32_t>(high) << 16)));
-      }
+      for (int dt = 0; dt < DT; ++dt) ks[dt] = load_bf16x8(kp + dt * 32);
       const bf16_t* vp = v_pages + ((page * kv_heads + kvh) * VDIM + col) * page_size + o0 + grp * 4;
-      const int beyond = j0 + grp * 4 + 3 - p_last;      // this many of the lane's four keys are not written yet
 #pragma unroll
-      for (int vt = 0; vt < VT; ++vt) {
-        short4_t values = load_bf16x4(vp + static_cast<long>(vt) * 16 * page_size);
-        if (beyond > 0) {
+      for (int vt = 0; vt < VT; ++vt) vs[vt] = load_bf16x4(vp + static_cast<long>(vt) * 16 * page_size);
+      return true;
+    };
+    const int j_first = lo_run & ~15;
+    there = fetch(j_first, keys, values);
+    for (int j0 = j_first; j0 <= p_last; j0 += 16) {
+      there_next = j0 + 16 <= p_last ? fetch(j0 + 16, keys_next, values_next) : false;
+      if (there) {
+        float4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-          for (int i = 0; i < 4; ++i)
-            if (i > 3 - beyond) values[i] = 0;
+        for (int dt = 0; dt < DT; ++dt)
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, keys[dt]),
+                                                        __builtin_bit_cast(bf16x8_t, qb[dt]), acc, 0, 0, 0);
+        float s[4];
+        float highest = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int j = j0 + grp * 4 + i;
+          float v = acc[i] * scale;
+          if (softcap > 0.f) v = softcap * tanhf(v / softcap);
+          s[i] = (in_run && j >= my_lowest && j <= my_pos) ? v : -INFINITY;
+          highest = fmaxf(highest, s[i]);
         }
-        float4_t sum = o[vt];
+        highest = fmaxf(highest, __shfl_xor(highest, 16, kWave));
+        highest = fmaxf(highest, __shfl_xor(highest, 32, kWave));
+        const float m_new = fmaxf(m, highest);
+        const float correction = m_new == m ? 1.f : expf(m - m_new);
+        float p[4], added = 0.f;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) sum[i] *= correction;
-        sum = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(values, p_high, sum, 0, 0, 0);
-        o[vt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(values, p_low, sum, 0, 0, 0);
+        for (int i = 0; i < 4; ++i) {
+          p[i] = s[i] == -INFINITY ? 0.f : expf(s[i] - m_new);
+          added += p[i];
+        }
+        added += __shfl_xor(added, 16, kWave);
+        added += __shfl_xor(added, 32, kWave);
+        l = l * correction + added;
+        m = m_new;
+        short4_t p_high, p_low;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const uint16_t high = bf16_bits(p[i]);
+          p_high[i] = static_cast<short>(high);
+          p_low[i] = static_cast<short>(bf16_bits(p[i] - __uint_as_float(static_cast<uint32_t>(high) << 16)));
+        }
+        const int beyond = j0 + grp * 4 + 3 - p_last;      // this many of the lane's four keys are not written yet
+#pragma unroll
+        for (int vt = 0; vt < VT; ++vt) {
+          short4_t operand = values[vt];
+          if (beyond > 0) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              if (i > 3 - beyond) operand[i] = 0;
+          }
+          float4_t sum = o[vt];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) sum[i] *= correction;
+          sum = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(operand, p_high, sum, 0, 0, 0);
+          o[vt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(operand, p_low, sum, 0, 0, 0);
+        }
       }
+      there = there_next;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) keys[dt] = keys_next[dt];
+#pragma unroll
+      for (int vt = 0; vt < VT; ++vt) values[vt] = values_next[vt];
     }
     row = run_end;
   }
   if (!have) return;
-  float gate = 1.f;
-  if (gates != nullptr) gate = 1.f / (1.f + expf(-to_float(gates[static_cast<long>(my_row) * gate_stride + gate_at + head])));
+  float gate = out_scale;
+  if (gates != nullptr) gate = out_scale / (1.f + expf(-to_float(gates[static_cast<long>(my_row) * gate_stride + gate_at + head])));
   const float factor = gate / l;
-  bf16_t* dst = out + (static_cast<long>(my_row) * q_heads + head) * VDIM + grp * 4;
+  bf16_t* dst = out + static_cast<long>(my_row) * out_stride + head * VDIM + grp * 4;
 #pragma unroll
   for (int vt = 0; vt < VT; ++vt) {
     uint2 packed;
@@ -291,7 +319,8 @@ int akv_gated_attention_tiles(const void* q, const void* k_pages, const void* v_
                               int gate_at, const int* seq_of_token, const int* q_start, const int* positions,
                               const int* block_table, const int* table_rows, int table_width, void* out, int first_row,
                               int tokens, int q_heads, int kv_heads, int dim, int vdim, int page_size, long num_pages,
-                              float scale, float softcap, int chunk, int window, int sink, hipStream_t stream) {
+                              float scale, float softcap, int chunk, int window, int sink, long out_stride, float out_scale,
+                              hipStream_t stream) {
   if (tokens <= first_row) return 0;
   if (page_size % 16 != 0 || q_heads % kv_heads != 0) return -2;
   const long items = static_cast<long>((tokens - first_row + 15) / 16) * q_heads;
@@ -301,7 +330,7 @@ int akv_gated_attention_tiles(const void* q, const void* k_pages, const void* v_
       static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_pages), static_cast<const bf16_t*>(v_pages),         \
       static_cast<const bf16_t*>(gates), gate_stride, gate_at, seq_of_token, q_start, positions, block_table, table_rows, \
       table_width, static_cast<bf16_t*>(out), first_row, tokens, q_heads, kv_heads, page_size, num_pages, scale, softcap, \
-      chunk, window, sink)
+      chunk, window, sink, out_stride, out_scale)
 #define AKV_TILES_V(DT)                    \
   switch (vdim) {                          \
     case 32: AKV_TILES(DT, 2); break;      \
@@ -311,10 +340,10 @@ int akv_gated_attention_tiles(const void* q, const void* k_pages, const void* v_
     default: return -2;                    \
   }
   switch (dim) {
-    case 32: AKV_TILES_V(2); break;
-    case 64: AKV_TILES_V(4); break;
-    case 128: AKV_TILES_V(8); break;
-    case 256: AKV_TILES_V(16); break;
+    case 32: AKV_TILES_V(1); break;
+    case 64: AKV_TILES_V(2); break;
+    case 128: AKV_TILES_V(4); break;
+    case 256: AKV_TILES_V(8); break;
     default: return -2;
   }
 #undef AKV_TILES_V
@@ -339,7 +368,7 @@ int akv_gated_attention_rows(const void* q, const void* k_pages, const void* v_p
                              int gate_at, const int* seq_of_token, const int* positions, const int* block_table,
                              const int* table_rows, int table_width, void* out, int dtype, long tokens, int q_heads,
                              int kv_heads, int dim, int vdim, int page_size, long num_pages, float scale, float softcap,
-                             int chunk, int window, int sink, hipStream_t stream) {
+                             int chunk, int window, int sink, long out_stride, float out_scale, hipStream_t stream) {
   if (tokens <= 0) return 0;
   if (vdim > kMaxValueRegs * kWave || dim <= 0 || q_heads % kv_heads != 0) return -2;
   const long rows = tokens * q_heads;
@@ -351,7 +380,7 @@ int akv_gated_attention_rows(const void* q, const void* k_pages, const void* v_p
                    static_cast<const T*>(q), static_cast<const T*>(k_pages), static_cast<const T*>(v_pages),
                    static_cast<const T*>(gates), gate_stride, gate_at, seq_of_token, positions, block_table, table_rows,
                    table_width, static_cast<T*>(out), tokens, q_heads, kv_heads, dim, vdim, page_size, num_pages, scale,
-                   softcap, chunk, window, sink));
+                   softcap, chunk, window, sink, out_stride, out_scale));
   return AKV_LAUNCH_STATUS();
 }
 }

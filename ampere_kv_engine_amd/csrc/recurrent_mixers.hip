@@ -28,7 +28,7 @@ __global__ __launch_bounds__(1024) void retention_kernel(
     const T* __restrict__ projected, long stride, int heads, int dim, int vdim, int rot_dims,
     const float* __restrict__ table, int table_positions, float key_scale, const float* __restrict__ decay, float eps,
     float* __restrict__ state, long state_stride, const int* __restrict__ q_start, const int* __restrict__ seq_slots,
-    const int* __restrict__ positions, T* __restrict__ out, int parts, int batch) {
+    const int* __restrict__ positions, T* __restrict__ out, int parts, int batch, long out_stride, float out_scale) {
   extern __shared__ float lds[];
   const int seq = blockIdx.x, h = blockIdx.y;
   const int tid = threadIdx.x, threads = blockDim.x;
@@ -105,7 +105,7 @@ __global__ __launch_bounds__(1024) void retention_kernel(
       const long n = first + base + t;
       for (int c = lane; c < vdim; c += kWave) {
         const float g = to_float(projected[n * stride + g_at + c]);
-        out[n * heads * vdim + static_cast<long>(h) * vdim + c] = from_float<T>(os[t * vdim + c] * scale * silu(g));
+        out[n * out_stride + static_cast<long>(h) * vdim + c] = from_float<T>(os[t * vdim + c] * scale * silu(g) * out_scale);
       }
     }
     __syncthreads();
@@ -177,11 +177,31 @@ __global__ __launch_bounds__(256) void retention_chunk_sums_kernel(
   for (int j = threadIdx.x; j < n; j += blockDim.x) ws[j] = power(w, n - 1 - j);
   __syncthreads();
   float* mine = sums + ((static_cast<long>(seq) * heads + h) * chunks + chunk) * dim * vdim;
-  for (int item = threadIdx.x; item < dim * vdim; item += blockDim.x) {
-    const int d = item / vdim, v = item % vdim;
-    float total = 0.f;
-    for (int j = 0; j < n; ++j) total = fmaf(ws[j] * ks[j * pitch + d], vs[j * vdim + v], total);
-    mine[item] = total;
+  // a thread owns patches of 8 x 8 of U: a token's 8 keys and 8 values from LDS feed 64 multiply-adds
+  const int across = (vdim + 7) / 8, patches = ((dim + 7) / 8) * across;
+  for (int patch = threadIdx.x; patch < patches; patch += blockDim.x) {
+    const int d0 = patch / across * 8, v0 = patch % across * 8;
+    float total[8][8];
+#pragma unroll
+    for (int a = 0; a < 8; ++a)
+#pragma unroll
+      for (int b = 0; b < 8; ++b) total[a][b] = 0.f;
+    for (int j = 0; j < n; ++j) {
+      float kd[8], vv[8];
+#pragma unroll
+      for (int a = 0; a < 8; ++a) kd[a] = d0 + a < dim ? ws[j] * ks[j * pitch + d0 + a] : 0.f;
+#pragma unroll
+      for (int b = 0; b < 8; ++b) vv[b] = v0 + b < vdim ? vs[j * vdim + v0 + b] : 0.f;
+#pragma unroll
+      for (int a = 0; a < 8; ++a)
+#pragma unroll
+        for (int b = 0; b < 8; ++b) total[a][b] = fmaf(kd[a], vv[b], total[a][b]);
+    }
+#pragma unroll
+    for (int a = 0; a < 8; ++a)
+#pragma unroll
+      for (int b = 0; b < 8; ++b)
+        if (d0 + a < dim && v0 + b < vdim) mine[static_cast<long>(d0 + a) * vdim + v0 + b] = total[a][b];
   }
 }
 
@@ -210,12 +230,12 @@ __global__ __launch_bounds__(256) void retention_chunk_states_kernel(const float
   *kept = S;
 }
 
-template <typename T>
+template <typename T, int GROUPS>
 __global__ __launch_bounds__(256) void retention_chunk_outputs_kernel(
     const T* __restrict__ projected, long stride, int heads, int dim, int vdim, int rot_dims,
     const float* __restrict__ table, int table_positions, float key_scale, const float* __restrict__ decay, float eps,
     const int* __restrict__ q_start, const int* __restrict__ positions, const float* __restrict__ states, int length,
-    int chunks, T* __restrict__ out) {
+    int chunks, T* __restrict__ out, long out_stride, float out_scale) {
   extern __shared__ float lds[];
   const int seq = blockIdx.x, h = blockIdx.y, chunk = blockIdx.z;
   const int first = q_start[seq], count = q_start[seq + 1] - first;
@@ -244,12 +264,41 @@ __global__ __launch_bounds__(256) void retention_chunk_outputs_kernel(
   }
   __syncthreads();
   const float* before = states + ((static_cast<long>(seq) * heads + h) * chunks + chunk) * dim * vdim;
-  for (int item = threadIdx.x; item < n * vdim; item += blockDim.x) {
-    const int t = item / vdim, v = item % vdim;
-    float carried = 0.f, within = 0.f;
-    for (int d = 0; d < dim; ++d) carried = fmaf(qs[t * pitch + d], before[static_cast<long>(d) * vdim + v], carried);
-    for (int j = 0; j <= t; ++j) within = fmaf(as[t * (length + 1) + j], vs[j * vdim + v], within);
-    os[item] = fmaf(ws[t + 1], carried, within);
+  // a thread keeps a column v of the values and the tokens group, group + GROUPS, ...: what it reads of the state before
+  // the chunk and of the chunk's values it reads once for all its tokens
+  constexpr int TP = 32 / GROUPS;
+  const int lanes = 256 / GROUPS, group = threadIdx.x / lanes;
+  for (int v = threadIdx.x % lanes; v < vdim; v += lanes) {
+    float carried[TP], within[TP];
+#pragma unroll
+    for (int k = 0; k < TP; ++k) carried[k] = within[k] = 0.f;
+    for (int d0 = 0; d0 < dim; d0 += 8) {       // eight rows of the state are asked for before the first is used
+      float held[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) held[e] = d0 + e < dim ? before[static_cast<long>(d0 + e) * vdim + v] : 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int d = min(d0 + e, dim - 1);
+#pragma unroll
+        for (int k = 0; k < TP; ++k) {
+          const int t = min(group + k * GROUPS, length - 1);      // (rows beyond the chunk's tokens count for nothing)
+          carried[k] = fmaf(qs[t * pitch + d], held[e], carried[k]);
+        }
+      }
+    }
+    for (int j = 0; j < n; ++j) {
+      const float value = vs[j * vdim + v];
+#pragma unroll
+      for (int k = 0; k < TP; ++k) {
+        const int t = group + k * GROUPS;
+        if (t < n && j <= t) within[k] = fmaf(as[t * (length + 1) + j], value, within[k]);
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < TP; ++k) {
+      const int t = group + k * GROUPS;
+      if (t < n) os[t * vdim + v] = fmaf(ws[t + 1], carried[k], within[k]);
+    }
   }
   __syncthreads();
   const int waves = blockDim.x / kWave, wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
@@ -261,13 +310,14 @@ __global__ __launch_bounds__(256) void retention_chunk_outputs_kernel(
     const long row = row0 + t;
     for (int c = lane; c < vdim; c += kWave) {
       const float g = to_float(projected[row * stride + g_at + c]);
-      out[row * heads * vdim + static_cast<long>(h) * vdim + c] = from_float<T>(os[t * vdim + c] * scale * silu(g));
+      out[row * out_stride + static_cast<long>(h) * vdim + c] = from_float<T>(os[t * vdim + c] * scale * silu(g) * out_scale);
     }
   }
 }
 
 // ---- gated linear recurrence ------------------------------------------------------------------------------------------
-// A block is a request and 64 neighbouring channels; its waves cut the request's tokens of this step into as many runs.
+// A block is a request and `ch` neighbouring channels (64, or 16 where runs are many); its threads cut the request's
+// tokens of this step into blockDim.x / ch runs.
 // Thread (run, channel) first takes its run from a state of zero - which gives the run's product of decays and what the
 // run adds -, the runs' pairs meet in LDS, every thread folds the pairs of the runs before its own onto the request's
 // state, and takes its run again from there, now writing S * gelu_tanh(y).  Tokens eight at a time: everything that
@@ -277,11 +327,11 @@ __global__ __launch_bounds__(1024) void gated_linear_scan_kernel(
     const T* __restrict__ u, const float* __restrict__ gates, const float* __restrict__ gate_bias,
     const float* __restrict__ rate, const T* __restrict__ y, long y_stride, int channels, int block_width,
     float* __restrict__ state, long state_stride, const int* __restrict__ q_start, const int* __restrict__ seq_slots,
-    T* __restrict__ out) {
-  __shared__ float products[16][kWave], sums[16][kWave];
+    T* __restrict__ out, int ch) {
+  __shared__ float products[1024], sums[1024];
   const int seq = blockIdx.x;
-  const int lane = threadIdx.x & (kWave - 1), run = threadIdx.x / kWave, runs = blockDim.x / kWave;
-  const int c = blockIdx.y * kWave + lane;
+  const int lane = threadIdx.x % ch, run = threadIdx.x / ch, runs = blockDim.x / ch;
+  const int c = blockIdx.y * ch + lane;
   const bool live = c < channels;
   const int first = q_start[seq], count = q_start[seq + 1] - first;
   const int per_run = (count + runs - 1) / runs;
@@ -325,14 +375,58 @@ __global__ __launch_bounds__(1024) void gated_linear_scan_kernel(
       }
     }
     if (pass == 0) {
-      products[run][lane] = product;
-      sums[run][lane] = S;
+      products[run * ch + lane] = product;
+      sums[run * ch + lane] = S;
       __syncthreads();
       S = *mine;
-      for (int before = 0; before < run; ++before) S = fmaf(products[before][lane], S, sums[before][lane]);
+      for (int before = 0; before < run; ++before) S = fmaf(products[before * ch + lane], S, sums[before * ch + lane]);
     }
   }
   if (run == runs - 1 && live) *mine = S;
+}
+
+template <typename T, int GROUPS>
+int launch_retention_outputs(const dim3 grid, size_t lds, hipStream_t stream, const T* projected, long stride, int heads, int dim,
+                             int vdim, int rot_dims, const float* table, int table_positions, float key_scale,
+                             const float* decay, float eps, const int* q_start, const int* positions, const float* states,
+                             int length, int chunks, T* out, long out_stride, float out_scale) {
+  if (lds > 64 * 1024 &&
+      hipFuncSetAttribute(reinterpret_cast<const void*>(&retention_chunk_outputs_kernel<T, GROUPS>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)) != hipSuccess)
+    return -2;
+  retention_chunk_outputs_kernel<T, GROUPS><<<grid, 256, lds, stream>>>(projected, stride, heads, dim, vdim, rot_dims, table,
+                                                                        table_positions, key_scale, decay, eps, q_start,
+                                                                        positions, states, length, chunks, out, out_stride,
+                                                                        out_scale);
+  return 0;
+}
+
+template <typename T>
+int launch_retention_chunked(const T* projected, long stride, int seqs, int heads, int dim, int vdim, int rot_dims,
+                             const float* table, int table_positions, float key_scale, const float* decay, float eps,
+                             float* state, long state_stride, const int* q_start, const int* seq_slots, const int* positions,
+                             T* out, long out_stride, float out_scale, float* sums, float* states, int length, int chunks,
+                             size_t lds_sums, size_t lds_outputs, hipStream_t stream) {
+  const dim3 grid(seqs, heads, chunks);
+  const int size = dim * vdim;
+  if (lds_sums > 64 * 1024 &&
+      hipFuncSetAttribute(reinterpret_cast<const void*>(&retention_chunk_sums_kernel<T>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_sums)) != hipSuccess)
+    return -2;
+  retention_chunk_sums_kernel<T><<<grid, 256, lds_sums, stream>>>(projected, stride, heads, dim, vdim, rot_dims, table,
+                                                                table_positions, key_scale, decay, q_start, positions, sums,
+                                                                length, chunks);
+  retention_chunk_states_kernel<<<dim3(seqs, heads, (size + 255) / 256), 256, 0, stream>>>(
+      sums, states, state, state_stride, decay, q_start, seq_slots, heads, size, length, chunks);
+#define AKV_OUTPUTS(GROUPS)                                                                                               \
+  launch_retention_outputs<T, GROUPS>(grid, lds_outputs, stream, projected, stride, heads, dim, vdim, rot_dims, table,       \
+                                      table_positions, key_scale, decay, eps, q_start, positions, states, length, chunks, out, \
+                                      out_stride, out_scale)
+  if (vdim <= 32) return AKV_OUTPUTS(8);
+  if (vdim <= 64) return AKV_OUTPUTS(4);
+  if (vdim <= 128) return AKV_OUTPUTS(2);
+  return AKV_OUTPUTS(1);
+#undef AKV_OUTPUTS
 }
 
 }  // namespace
@@ -342,7 +436,7 @@ extern "C" {
 int akv_retention(const void* projected, long stride, int dtype, int seqs, int heads, int dim, int vdim, int rot_dims,
                   const float* table, int table_positions, float key_scale, const float* decay, float eps, float* state,
                   long state_stride, const int* q_start, const int* seq_slots, const int* positions, void* out,
-                  hipStream_t stream) {
+                  long out_stride, float out_scale, hipStream_t stream) {
   if (seqs <= 0) return 0;
   if (heads <= 0 || dim <= 0 || vdim <= 0 || vdim > 1024 || rot_dims < 0 || rot_dims % 2 || rot_dims > dim) return -2;
   if (rot_dims > 0 && (table == nullptr || table_positions <= 0)) return -2;
@@ -365,7 +459,7 @@ int akv_retention(const void* projected, long stride, int dtype, int seqs, int h
   AKV_DISPATCH(dtype, T, retention_kernel<T, R><<<grid, threads, lds_of(batch), stream>>>(                             \
                              static_cast<const T*>(projected), stride, heads, dim, vdim, rot_dims, table, table_positions, \
                              key_scale, decay, eps, state, state_stride, q_start, seq_slots, positions,                 \
-                             static_cast<T*>(out), parts, batch))
+                             static_cast<T*>(out), parts, batch, out_stride, out_scale))
   switch (per_thread) {
     case 4: AKV_RETENTION(4); break;
     case 8: AKV_RETENTION(8); break;
@@ -382,35 +476,22 @@ int akv_retention(const void* projected, long stride, int dtype, int seqs, int h
 int akv_retention_chunked(const void* projected, long stride, int dtype, int seqs, int heads, int dim, int vdim, int rot_dims,
                           const float* table, int table_positions, float key_scale, const float* decay, float eps,
                           float* state, long state_stride, const int* q_start, const int* seq_slots, const int* positions,
-                          void* out, float* sums, int length, int chunks, hipStream_t stream) {
+                          void* out, long out_stride, float out_scale, float* sums, int length, int chunks,
+                          hipStream_t stream) {
   if (seqs <= 0 || chunks <= 0) return 0;
-  if (heads <= 0 || dim <= 0 || vdim <= 0 || rot_dims < 0 || rot_dims % 2 || rot_dims > dim || length < 1) return -2;
+  if (heads <= 0 || dim <= 0 || vdim <= 0 || rot_dims < 0 || rot_dims % 2 || rot_dims > dim || length < 1 || length > 32) return -2;
   if (rot_dims > 0 && (table == nullptr || table_positions <= 0)) return -2;
   const int pitch = dim + 1;
   const size_t lds_sums = static_cast<size_t>(length * pitch + length * vdim + length) * 4;
   const size_t lds_outputs = static_cast<size_t>(2 * length * pitch + 2 * length * vdim + length * (length + 1) + length + 1) * 4;
   if (lds_sums > 128 * 1024 || lds_outputs > 128 * 1024) return -2;
-  const dim3 grid(seqs, heads, chunks);
-  const int size = dim * vdim;
-  float* states = sums + static_cast<long>(seqs) * heads * chunks * size;
-  AKV_DISPATCH(dtype, T, {
-    if (lds_sums > 64 * 1024 &&
-        hipFuncSetAttribute(reinterpret_cast<const void*>(&retention_chunk_sums_kernel<T>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_sums)) != hipSuccess)
-      return -2;
-    if (lds_outputs > 64 * 1024 &&
-        hipFuncSetAttribute(reinterpret_cast<const void*>(&retention_chunk_outputs_kernel<T>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_outputs)) != hipSuccess)
-      return -2;
-    retention_chunk_sums_kernel<T><<<grid, 256, lds_sums, stream>>>(static_cast<const T*>(projected), stride, heads, dim, vdim,
-                                                                  rot_dims, table, table_positions, key_scale, decay, q_start,
-                                                                  positions, sums, length, chunks);
-    retention_chunk_states_kernel<<<dim3(seqs, heads, (size + 255) / 256), 256, 0, stream>>>(
-        sums, states, state, state_stride, decay, q_start, seq_slots, heads, size, length, chunks);
-    retention_chunk_outputs_kernel<T><<<grid, 256, lds_outputs, stream>>>(
-        static_cast<const T*>(projected), stride, heads, dim, vdim, rot_dims, table, table_positions, key_scale, decay, eps,
-        q_start, positions, states, length, chunks, static_cast<T*>(out));
-  });
+  float* states = sums + static_cast<long>(seqs) * heads * chunks * dim * vdim;
+  int status = 0;
+  AKV_DISPATCH(dtype, T, status = launch_retention_chunked<T>(
+                             static_cast<const T*>(projected), stride, seqs, heads, dim, vdim, rot_dims, table, table_positions,
+                             key_scale, decay, eps, state, state_stride, q_start, seq_slots, positions, static_cast<T*>(out),
+                             out_stride, out_scale, sums, states, length, chunks, lds_sums, lds_outputs, stream));
+  if (status != 0) return status;
   return AKV_LAUNCH_STATUS();
 }
 
@@ -418,11 +499,12 @@ int akv_gated_linear_scan(const void* u, int dtype, const float* gates, const fl
                           const void* y, long y_stride, int seqs, int channels, int blocks, int runs, float* state,
                           long state_stride, const int* q_start, const int* seq_slots, void* out, hipStream_t stream) {
   if (seqs <= 0) return 0;
-  if (channels <= 0 || blocks <= 0 || channels % blocks || runs < 1 || runs > 16) return -2;
-  const dim3 grid(seqs, (channels + kWave - 1) / kWave);
-  AKV_DISPATCH(dtype, T, gated_linear_scan_kernel<T><<<grid, runs * kWave, 0, stream>>>(
+  if (channels <= 0 || blocks <= 0 || channels % blocks || runs < 1 || runs > 64) return -2;
+  const int ch = runs > 16 ? 16 : kWave;
+  const dim3 grid(seqs, (channels + ch - 1) / ch);
+  AKV_DISPATCH(dtype, T, gated_linear_scan_kernel<T><<<grid, runs * ch, 0, stream>>>(
                              static_cast<const T*>(u), gates, gate_bias, rate, static_cast<const T*>(y), y_stride, channels,
-                             channels / blocks, state, state_stride, q_start, seq_slots, static_cast<T*>(out)));
+                             channels / blocks, state, state_stride, q_start, seq_slots, static_cast<T*>(out), ch));
   return AKV_LAUNCH_STATUS();
 }
 }

@@ -22,6 +22,11 @@ def _long(value: int):
     return ctypes.c_long(int(value))
 
 
+def _ptr_at(t, column: int):
+    """Where column `column` of the first row of a dense [rows, width] tensor lies."""
+    return ctypes.c_void_p(t.data_ptr() + int(column) * t.element_size())
+
+
 class PartsKernels:
     """Mixed into `HipKernels` (which provides `_dense`, `_check`, `_stream`, `device`)."""
 
@@ -404,30 +409,33 @@ class PartsKernels:
         self._dense(v_pages, "v_pages", dtype, (k_pages.shape[0], kv_heads, vdim, k_pages.shape[2]))
         return k_pages.shape[0], k_pages.shape[2]
 
-    def unit_norm_write(self, projected, q_heads, kv_heads, dim, vdim, eps, slot_map, k_pages, v_pages, q_out) -> None:
-        """projected [tokens, q | k | v | ...]: the query heads divided by their root mean square (eps inside the root;
+    def unit_norm_write(self, projected, q_heads, kv_heads, dim, vdim, eps, slot_map, k_pages, v_pages, q_out, at: int = 0) -> None:
+        """projected [tokens, ... | q | k | v | ...] with q at column `at`: the query heads divided by their root mean square (eps inside the root;
         `eps` None: as they are) -> q_out; with `slot_map` the key heads, the same way, and the value heads into the
         tokens' slots of the pages."""
         tokens = projected.shape[0]
         self._dense(projected, "projected")
-        if projected.dim() != 2 or projected.shape[1] < (q_heads + kv_heads) * dim + kv_heads * vdim:
+        if projected.dim() != 2 or at < 0 or projected.shape[1] < at + (q_heads + kv_heads) * dim + kv_heads * vdim:
             self._refuse(f"projected rows must hold queries, keys and values, got {tuple(projected.shape)}")
         self._dense(q_out, "q_out", projected.dtype, (tokens, q_heads * dim))
         num_pages, page_size = self._gated_pages(k_pages, v_pages, kv_heads, dim, vdim, projected.dtype)
         if slot_map is not None:
             self._dense(slot_map, "slot_map", torch.int32, (tokens,))
         self._check(self._parts().akv_unit_norm_write(
-            _ptr(projected), _long(projected.shape[1]), self._code_of(projected), _long(tokens), q_heads, kv_heads, dim, vdim,
-            ctypes.c_float(eps if eps is not None else 0.0), 0 if eps is None else 1, _ptr(slot_map), _ptr(k_pages),
+            _ptr_at(projected, at), _long(projected.shape[1]), self._code_of(projected), _long(tokens), q_heads, kv_heads, dim,
+            vdim, ctypes.c_float(eps if eps is not None else 0.0), 0 if eps is None else 1, _ptr(slot_map), _ptr(k_pages),
             _ptr(v_pages), page_size, _long(num_pages), _ptr(q_out), self._stream()), "unit_norm_write")
 
     def gated_attention(self, q, k_pages, v_pages, gates, gate_at, ctx, meta, q_heads, kv_heads, dim, vdim, scale, softcap,
-                        chunk, window, sink, out) -> None:
-        """Every query head attends the keys of its request that it sees (see `parts/gated_attention.py`) -> out
-        [tokens, q_heads * vdim]; `gates` [tokens, width]: head h's output times sigmoid(gates[t, gate_at + h])."""
+                        chunk, window, sink, out, out_at: int = 0, out_scale: float = 1.0) -> None:
+        """Every query head attends the keys of its request that it sees (see `parts/gated_attention.py`) -> columns
+        out_at .. out_at + q_heads * vdim of `out`, times `out_scale`; `gates` [tokens, width]: head h's output times
+        sigmoid(gates[t, gate_at + h])."""
         tokens = q.shape[0]
         self._dense(q, "q", None, (tokens, q_heads * dim))
-        self._dense(out, "out", q.dtype, (tokens, q_heads * vdim))
+        self._dense(out, "out", q.dtype)
+        if out.dim() != 2 or out.shape[0] != tokens or out_at < 0 or out_at + q_heads * vdim > out.shape[1]:
+            self._refuse(f"out must be [tokens, at least {out_at + q_heads * vdim}], got {tuple(out.shape)}")
         num_pages, page_size = self._gated_pages(k_pages, v_pages, kv_heads, dim, vdim, q.dtype)
         gate_stride = 0
         if gates is not None:
@@ -449,34 +457,40 @@ class PartsKernels:
             self._refuse("a request is longer than its row of the block table")
         tail = (ctypes.c_float(scale), ctypes.c_float(softcap if softcap is not None else 0.0),
                 int(chunk) if chunk is not None else 0, int(window) if window is not None else 0, 1 if sink else 0,
-                self._stream())
+                _long(out.shape[1]), ctypes.c_float(out_scale), self._stream())
         singles = tokens
         if (q.dtype == torch.bfloat16 and dim in self.MATRIX_CORE_HEAD_DIMS and vdim in self.MATRIX_CORE_HEAD_DIMS
-                and page_size % 16 == 0):
+                and page_size % 16 == 0 and out.shape[1] % 4 == 0 and out_at % 4 == 0):
             # single tokens: a wave per token and head; the portions' rows, which follow them, go to the matrix cores
             singles = ctx.num_decode_seqs
             self._check(self._parts().akv_gated_attention_tiles(
                 _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(gates), _long(gate_stride), gate_at, _ptr(ctx.seq_of_token),
-                _ptr(ctx.q_start), _ptr(ctx.positions), _ptr(meta.block_table), _ptr(meta.rows), meta.width, _ptr(out),
-                singles, tokens, q_heads, kv_heads, dim, vdim, page_size, _long(num_pages), *tail),
+                _ptr(ctx.q_start), _ptr(ctx.positions), _ptr(meta.block_table), _ptr(meta.rows), meta.width,
+                _ptr_at(out, out_at), singles, tokens, q_heads, kv_heads, dim, vdim, page_size, _long(num_pages), *tail),
                 "gated_attention on the matrix cores")
         if singles:
             self._check(self._parts().akv_gated_attention_rows(
                 _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(gates), _long(gate_stride), gate_at, _ptr(ctx.seq_of_token),
-                _ptr(ctx.positions), _ptr(meta.block_table), _ptr(meta.rows), meta.width, _ptr(out), self._code_of(q),
-                _long(singles), q_heads, kv_heads, dim, vdim, page_size, _long(num_pages), *tail), "gated_attention")
+                _ptr(ctx.positions), _ptr(meta.block_table), _ptr(meta.rows), meta.width, _ptr_at(out, out_at),
+                self._code_of(q), _long(singles), q_heads, kv_heads, dim, vdim, page_size, _long(num_pages), *tail), "gated_attention")
 
     # ---- mixers with a state of fixed size -----------------------------------------------------------------------------
     def check_retention_sizes(self, heads: int, dim: int, vdim: int) -> None:
         if not 0 < vdim <= 1024 or dim <= 0 or vdim * ((dim + 63) // 64) > 1024:
             self._refuse(f"retention keeps a head's state [{dim}, {vdim}] in one block's registers: up to 65,536 values")
 
-    def retention(self, projected, heads, dim, vdim, rot_dims, table, key_scale, decay, eps, state, ctx, out) -> None:
-        """projected [tokens, q | k | v | g] -> out [tokens, heads * vdim] = (S^T q) / rms * silu(g) with S <- decay S +
-        k v^T per request and head (see `parts/retention.py`); S lies in the request's slot of `state`, float32."""
+    def retention(self, projected, heads, dim, vdim, rot_dims, table, key_scale, decay, eps, state, ctx, out, at: int = 0,
+                  out_at: int = 0, out_scale: float = 1.0) -> None:
+        """projected [tokens, ... | q | k | v | g | ...] with q at column `at` -> columns out_at .. out_at + heads * vdim of
+        `out` = (S^T q) / rms * silu(g) * out_scale with S <- decay S + k v^T per request and head (see
+        `parts/retention.py`); S lies in the request's slot of `state`, float32."""
         tokens = projected.shape[0]
-        self._dense(projected, "projected", None, (tokens, 2 * heads * (dim + vdim)))
-        self._dense(out, "out", projected.dtype, (tokens, heads * vdim))
+        self._dense(projected, "projected")
+        if projected.dim() != 2 or at < 0 or projected.shape[1] < at + 2 * heads * (dim + vdim):
+            self._refuse(f"projected rows must hold queries, keys, values and gates from column {at}, got {tuple(projected.shape)}")
+        self._dense(out, "out", projected.dtype)
+        if out.dim() != 2 or out.shape[0] != tokens or out_at < 0 or out_at + heads * vdim > out.shape[1]:
+            self._refuse(f"out must be [tokens, at least {out_at + heads * vdim}], got {tuple(out.shape)}")
         self._dense(decay, "decay", torch.float32, (heads,))
         self._dense(state, "state", torch.float32)
         if state.dim() != 2 or state.shape[1] != heads * dim * vdim:
@@ -490,10 +504,10 @@ class PartsKernels:
                 self._refuse(f"the rotation table must be [positions, {rot_dims // 2}, 2], got {tuple(table.shape)}")
             positions = table.shape[0]       # (the engine admits no request beyond the positions its tables were built for)
         self._step_arrays(ctx, tokens)
-        head = (_ptr(projected), _long(projected.shape[1]), self._code_of(projected), ctx.num_seqs, heads, dim, vdim, rot_dims,
-                _ptr(table) if rot_dims else ctypes.c_void_p(0), positions, ctypes.c_float(key_scale), _ptr(decay),
+        head = (_ptr_at(projected, at), _long(projected.shape[1]), self._code_of(projected), ctx.num_seqs, heads, dim, vdim,
+                rot_dims, _ptr(table) if rot_dims else ctypes.c_void_p(0), positions, ctypes.c_float(key_scale), _ptr(decay),
                 ctypes.c_float(eps), _ptr(state), _long(state.shape[1]), _ptr(ctx.q_start), _ptr(ctx.seq_slots),
-                _ptr(ctx.positions), _ptr(out))
+                _ptr(ctx.positions), _ptr_at(out, out_at), _long(out.shape[1]), ctypes.c_float(out_scale))
         length = self._retention_chunk(dim, vdim)
         if ctx.max_new_tokens >= self.RETENTION_CHUNKED_FROM and length:
             # portions: chunks side by side (the step's shape alone decides, so a recorded step replays the same launches)
@@ -526,9 +540,9 @@ class PartsKernels:
 
     @staticmethod
     def _scan_runs(longest_portion: int) -> int:
-        """Runs that the longest portion of a step is cut into: about 32 tokens a run, 16 runs at most (the step's shape
+        """Runs that the longest portion of a step is cut into: 16 tokens a run and more, 64 runs at most (the step's shape
         alone decides, so a recorded step is cut as the same step run eagerly)."""
-        return max(1, min(16, longest_portion // 32))
+        return max(1, min(64, longest_portion // 16))
 
     def gated_linear_scan(self, u, gates, gate_bias, rate, xy, blocks, state, taps, ctx, out) -> None:
         """Per request and channel, token after token: a = exp(rate * sigmoid(gates_r + bias)), S <- a S + sqrt(1 - a^2)

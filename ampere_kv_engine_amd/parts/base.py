@@ -177,6 +177,20 @@ class Part:
         return 0
 
 
+class SharesProducts:
+    """A mixer whose first step is one product over the layer's input (`inputs`, a `Linear` whose names are relative to
+    the mixer's own prefix) and whose last is one product (`outputs`) says so by deriving from this: side by side with
+    others of its kind (`parts/parallel.py`) all first products become one, all last ones one.  `attend_columns` does
+    everything between: it reads its columns of the shared projection (from column `at`) and leaves the rows its last
+    product would read in columns `out_at` on of `out`, times `out_scale`."""
+
+    inputs = None
+    outputs = None
+
+    def attend_columns(self, projected, at: int, ctx, cache, writes_cache: bool, out, out_at: int, out_scale: float) -> None:
+        raise NotImplementedError
+
+
 class Norm(Part):
     """What a block asks of a norm.  `forward` and `forward_residual` compute at once; `pending` and `scaled` offer
     the result before it is computed, for a reader whose first product can compute it (`UnnormedRows`) - None, the

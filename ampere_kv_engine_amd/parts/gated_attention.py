@@ -14,11 +14,11 @@ after their norm.  All five projections are one product over the layer's input.
 
 from __future__ import annotations
 
-from .base import PagedKV, Part, register_part
+from .base import PagedKV, Part, SharesProducts, register_part
 from .linear import Linear
 
 
-class GatedAttention(Part):
+class GatedAttention(Part, SharesProducts):
     graph_safe = True
 
     def __init__(self, spec, runtime):
@@ -53,8 +53,8 @@ class GatedAttention(Part):
             if biases:
                 biases.append(None)
         self.width = sum(sizes)
-        self.qkvg = Linear(runtime, self.hidden, sizes, stacked, bias_names=biases)
-        self.out = Linear(runtime, self.q_heads * self.vdim, [self.hidden], [names["o"]])
+        self.qkvg = self.inputs = Linear(runtime, self.hidden, sizes, stacked, bias_names=biases)
+        self.out = self.outputs = Linear(runtime, self.q_heads * self.vdim, [self.hidden], [names["o"]])
         runtime.kernels.check_gated_attention_sizes(self.q_heads, self.kv_heads, self.dim, self.vdim, runtime.page_size)
 
     def _prefix(self, prefix):
@@ -75,25 +75,25 @@ class GatedAttention(Part):
     def cache_request(self):
         return PagedKV(self.kv_heads, self.dim, self.window, value_dim=self.vdim, chunk=self.chunk)
 
-    def attend(self, x, ctx, cache, writes_cache: bool = True):
-        """x [tokens, hidden] -> the heads' gated outputs [tokens, q_heads * value_dim], before the output product."""
-        k, dtype = self.rt.kernels, self.rt.dtype
-        tokens = x.shape[0]
+    def attend_columns(self, projected, at, ctx, cache, writes_cache, out, out_at, out_scale):
+        """The heads' gated outputs, before the output product, from this mixer's columns of a projection."""
+        k = self.rt.kernels
         meta = ctx.paged[cache.group]
-        projected = ctx.arena.take((tokens, self.width), dtype)
-        self.qkvg.forward(x, projected)
-        q = ctx.arena.take((tokens, self.q_size), dtype)
+        q = ctx.arena.take((projected.shape[0], self.q_size), self.rt.dtype)
         k.unit_norm_write(projected, self.q_heads, self.kv_heads, self.dim, self.vdim, self.unit_eps,
-                          meta.slot_map if writes_cache else None, cache.k, cache.v, q)
-        merged = ctx.arena.take((tokens, self.q_heads * self.vdim), dtype)
+                          meta.slot_map if writes_cache else None, cache.k, cache.v, q, at=at)
         k.gated_attention(q, cache.k, cache.v, projected if self.head_gate else None,
-                          self.q_size + self.k_size + self.v_size, ctx, meta, self.q_heads, self.kv_heads, self.dim,
-                          self.vdim, self.scale, self.softcap, self.chunk, self.window, self.sink, merged)
-        return merged
+                          at + self.q_size + self.k_size + self.v_size, ctx, meta, self.q_heads, self.kv_heads, self.dim,
+                          self.vdim, self.scale, self.softcap, self.chunk, self.window, self.sink, out, out_at=out_at,
+                          out_scale=out_scale)
 
     def forward(self, x, ctx, cache, writes_cache: bool = True):
-        merged = self.attend(x, ctx, cache, writes_cache)
-        out = ctx.arena.take((x.shape[0], self.hidden), self.rt.dtype)
+        tokens, dtype = x.shape[0], self.rt.dtype
+        projected = ctx.arena.take((tokens, self.width), dtype)
+        self.qkvg.forward(x, projected)
+        merged = ctx.arena.take((tokens, self.q_heads * self.vdim), dtype)
+        self.attend_columns(projected, 0, ctx, cache, writes_cache, merged, 0, 1.0)
+        out = ctx.arena.take((tokens, self.hidden), dtype)
         return self.out.forward(merged, out)
 
 

@@ -15,11 +15,11 @@ from __future__ import annotations
 import numpy as np
 import torch
 
-from .base import Part, SlotState, register_part
+from .base import Part, SharesProducts, SlotState, register_part
 from .linear import Linear
 
 
-class Retention(Part):
+class Retention(Part, SharesProducts):
     graph_safe = True
 
     def __init__(self, spec, runtime):
@@ -38,8 +38,8 @@ class Retention(Part):
         names = dict(q="q", k="k", v="v", g="g", o="o")
         names.update(spec.get("names") or {})
         qk, vs = self.heads * self.dim, self.heads * self.vdim
-        self.qkvg = Linear(runtime, self.hidden, [qk, qk, vs, vs], [names["q"], names["k"], names["v"], names["g"]])
-        self.out = Linear(runtime, vs, [self.hidden], [names["o"]])
+        self.qkvg = self.inputs = Linear(runtime, self.hidden, [qk, qk, vs, vs], [names["q"], names["k"], names["v"], names["g"]])
+        self.out = self.outputs = Linear(runtime, vs, [self.hidden], [names["o"]])
         self.decay = torch.tensor(decay, dtype=torch.float32, device=runtime.device)
         self.table = None
         if self.rot_dims:
@@ -71,20 +71,18 @@ class Retention(Part):
     def cache_request(self):
         return SlotState((self.heads * self.dim * self.vdim,), torch.float32)
 
-    def attend(self, x, ctx, cache, writes_cache: bool = True):
-        """x [tokens, hidden] -> [tokens, heads * value_dim]: the heads' normed outputs times silu(W_g h), before W_o."""
-        k, dtype = self.rt.kernels, self.rt.dtype
-        tokens = x.shape[0]
+    def attend_columns(self, projected, at, ctx, cache, writes_cache, out, out_at, out_scale):
+        """The heads' normed outputs times silu(W_g h), before W_o, from this mixer's columns of a projection."""
+        self.rt.kernels.retention(projected, self.heads, self.dim, self.vdim, self.rot_dims, self.table, self.key_scale,
+                                  self.decay, self.eps, cache.state, ctx, out, at=at, out_at=out_at, out_scale=out_scale)
+
+    def forward(self, x, ctx, cache, writes_cache: bool = True):
+        tokens, dtype = x.shape[0], self.rt.dtype
         projected = ctx.arena.take((tokens, 2 * self.heads * (self.dim + self.vdim)), dtype)
         self.qkvg.forward(x, projected)
         gated = ctx.arena.take((tokens, self.heads * self.vdim), dtype)
-        k.retention(projected, self.heads, self.dim, self.vdim, self.rot_dims, self.table, self.key_scale, self.decay,
-                    self.eps, cache.state, ctx, gated)
-        return gated
-
-    def forward(self, x, ctx, cache, writes_cache: bool = True):
-        gated = self.attend(x, ctx, cache, writes_cache)
-        out = ctx.arena.take((x.shape[0], self.hidden), self.rt.dtype)
+        self.attend_columns(projected, 0, ctx, cache, writes_cache, gated, 0, 1.0)
+        out = ctx.arena.take((tokens, self.hidden), dtype)
         return self.out.forward(gated, out)
 
 

@@ -374,7 +374,8 @@ class TorchKernels(KernelSet):
     def check_retention_sizes(self, heads, dim, vdim):
         pass
 
-    def unit_norm_write(self, projected, q_heads, kv_heads, dim, vdim, eps, slot_map, k_pages, v_pages, q_out):
+    def unit_norm_write(self, projected, q_heads, kv_heads, dim, vdim, eps, slot_map, k_pages, v_pages, q_out, at=0):
+        projected = projected[:, at:]
         n = projected.shape[0]
         q_size, k_size, v_size = q_heads * dim, kv_heads * dim, kv_heads * vdim
         q = projected[:, :q_size].reshape(n, q_heads, dim).float()
@@ -391,7 +392,7 @@ class TorchKernels(KernelSet):
             v_pages[slots // page_size, :, :, slots % page_size] = v.to(v_pages.dtype)
 
     def gated_attention(self, q, k_pages, v_pages, gates, gate_at, ctx, meta, q_heads, kv_heads, dim, vdim, scale, softcap,
-                        chunk, window, sink, out):
+                        chunk, window, sink, out, out_at=0, out_scale=1.0):
         page_size = k_pages.shape[2]
         group = q_heads // kv_heads
         table = meta.block_table.cpu()
@@ -432,14 +433,15 @@ class TorchKernels(KernelSet):
                 merged[:, head] = (weights / total) @ values[:, head // group]
             if gates is not None:
                 merged = merged * torch.sigmoid(gates[first:last, gate_at:gate_at + q_heads].float())[:, :, None]
-            out[first:last] = merged.reshape(last - first, q_heads * vdim).to(out.dtype)
+            out[first:last, out_at:out_at + q_heads * vdim] = (merged.reshape(last - first, q_heads * vdim) * out_scale).to(out.dtype)
 
-    def retention(self, projected, heads, dim, vdim, rot_dims, table, key_scale, decay, eps, state, ctx, out):
+    def retention(self, projected, heads, dim, vdim, rot_dims, table, key_scale, decay, eps, state, ctx, out, at=0, out_at=0,
+                  out_scale=1.0):
         n = projected.shape[0]
         qk, vs = heads * dim, heads * vdim
-        p = projected.float()
+        p = projected[:, at:].float()
         q, k = p[:, :qk].reshape(n, heads, dim), p[:, qk:2 * qk].reshape(n, heads, dim)
-        v, g = p[:, 2 * qk:2 * qk + vs].reshape(n, heads, vdim), p[:, 2 * qk + vs:]
+        v, g = p[:, 2 * qk:2 * qk + vs].reshape(n, heads, vdim), p[:, 2 * qk + vs:2 * qk + 2 * vs]
         if rot_dims:
             q, k = self._turn(q, ctx.positions, table, rot_dims), self._turn(k, ctx.positions, table, rot_dims)
         k = k * key_scale
@@ -451,7 +453,7 @@ class TorchKernels(KernelSet):
                 o = torch.einsum("hdv,hd->hv", S, q[t])
                 o = o * torch.rsqrt((o * o).mean(-1, keepdim=True) + eps)
                 gate = g[t]
-                out[t] = (o.reshape(-1) * gate * torch.sigmoid(gate)).to(out.dtype)
+                out[t, out_at:out_at + vs] = (o.reshape(-1) * gate * torch.sigmoid(gate) * out_scale).to(out.dtype)
             state[slot] = S.reshape(-1)
 
     def scaled_sum(self, a, scale_a, b, scale_b, out):
