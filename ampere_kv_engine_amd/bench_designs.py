@@ -49,9 +49,9 @@ def keranex_config(size: dict, layers: int) -> dict:
 # unit + routed feed-forward, recurrent unit + dense, attention beside retention + routed]; a token uses `top` experts and
 # the shared one, as wide together as the dense feed-forward.
 TUKEVIK_SIZES = {
-    "s": dict(width=2048, vocab=32768, heads=16, kv_heads=4, dim=128, vdim=128, chunk=1024, r_heads=4, r_dim=128, r_vdim=128,
+    "s": dict(width=2048, vocab=32768, heads=16, kv_heads=4, dim=128, vdim=128, chunk=4096, r_heads=4, r_dim=128, r_vdim=128,
               recurrent=2048, blocks=16, conv=4, experts=16, top=2, ff=1024, shared=1024, dense=3072),
-    "m": dict(width=4096, vocab=65536, heads=32, kv_heads=8, dim=128, vdim=128, chunk=2048, r_heads=8, r_dim=128, r_vdim=128,
+    "m": dict(width=4096, vocab=65536, heads=32, kv_heads=8, dim=128, vdim=128, chunk=4096, r_heads=8, r_dim=128, r_vdim=128,
               recurrent=4096, blocks=16, conv=4, experts=32, top=4, ff=1024, shared=1024, dense=5120),
 }
 

@@ -40,11 +40,13 @@ int akv_unit_norm_write(const void* projected, long stride, int dtype, long toke
 // position p sees the keys j <= p with j > p - window (window > 0) and floor(j / chunk) = floor(p / chunk) (chunk > 0);
 // with `sink` the softmax's denominator has one more term exp(0); with `gates` head h's output is multiplied by
 // sigmoid(gates[t * gate_stride + gate_at + h]).  A token's outputs lie at out + t * out_stride, times out_scale.
+// `row_waves` (1 .. 16) waves share a token's head: each takes every row_waves-th tile of 64 keys.
 int akv_gated_attention_rows(const void* q, const void* k_pages, const void* v_pages, const void* gates, long gate_stride,
                              int gate_at, const int* seq_of_token, const int* positions, const int* block_table,
                              const int* table_rows, int table_width, void* out, int dtype, long tokens, int q_heads,
                              int kv_heads, int dim, int vdim, int page_size, long num_pages, float scale, float softcap,
-                             int chunk, int window, int sink, long out_stride, float out_scale, hipStream_t stream);
+                             int chunk, int window, int sink, long out_stride, float out_scale, int row_waves,
+                             hipStream_t stream);
 
 // The same for rows first_row .. tokens - 1 of a bfloat16 step, on the matrix cores: keys and values 32, 64, 128 or 256
 // wide, pages of a multiple of 16 tokens (-2 otherwise); a request's rows follow each other in the order of their positions.

@@ -68,22 +68,46 @@ __global__ __launch_bounds__(256) void unit_norm_write_kernel(const T* __restric
 }
 
 constexpr int kMaxValueRegs = 4;  // value widths up to 256: each lane owns dims lane, lane + 64, ...
+constexpr int kMaxRowWaves = 16;  // the most waves that share a (token, head): wave w of W takes the key tiles w, w + W, ...
 
-template <typename T>
-__global__ __launch_bounds__(256) void gated_attention_rows_kernel(
+// Eight bfloat16 (or float32) values from 16-byte aligned memory, widened.
+__device__ __forceinline__ void load8(const bf16_t* p, float (&v)[8]) {
+  const uint4 raw = *reinterpret_cast<const uint4*>(p);
+  const uint32_t words[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    v[2 * k] = __uint_as_float(words[k] << 16);
+    v[2 * k + 1] = __uint_as_float(words[k] & 0xffff0000u);
+  }
+}
+__device__ __forceinline__ void load8(const float* p, float (&v)[8]) {
+  const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+  v[0] = a.x, v[1] = a.y, v[2] = a.z, v[3] = a.w, v[4] = b.x, v[5] = b.y, v[6] = b.z, v[7] = b.w;
+}
+
+// A block is a (token, query head); its waves (1 to 16, the caller's choice) take the row's key tiles in turn and their shares - maximum, sum of
+// weights, weighted values - meet in LDS in the order of the waves.  Inside a tile a lane scores one key (VEC: its
+// dimensions eight at a time) and then owns value dimensions, for which it reads eight neighbouring keys' values at a
+// time (the value pages lie [vdim, page]).  VEC needs key rows and groups of eight values that are 16-byte aligned.
+template <typename T, bool VEC>
+__global__ __launch_bounds__(kMaxRowWaves * kWave) void gated_attention_rows_kernel(
     const T* __restrict__ q, const T* __restrict__ k_pages, const T* __restrict__ v_pages, const T* __restrict__ gates,
     long gate_stride, int gate_at, const int* __restrict__ seq_of_token, const int* __restrict__ positions,
     const int* __restrict__ block_table, const int* __restrict__ table_rows, int table_width, T* __restrict__ out,
     long tokens, int q_heads, int kv_heads, int dim, int vdim, int page_size, long num_pages, float scale, float softcap,
     int chunk, int window, int sink, long out_stride, float out_scale) {
   extern __shared__ unsigned char lds_raw[];
-  const int waves = blockDim.x / kWave, wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
-  const long row = static_cast<long>(blockIdx.x) * waves + wave;
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1), kRowWaves = blockDim.x / kWave;
+  // blocks go to the XCDs in turn: neighbouring rows - the query heads of one key head, which read the same keys and
+  // values - are given to blocks of one XCD, whose L2 then fetches those once
+  const long row = static_cast<long>(blockIdx.x % kXcds) * (gridDim.x / kXcds) + blockIdx.x / kXcds;
   if (row >= tokens * q_heads) return;
-  const size_t per_wave = (static_cast<size_t>(dim) * 4 + kWave * 4 + kWave * 8 + 7) / 8 * 8;
-  float* qs = reinterpret_cast<float*>(lds_raw + wave * per_wave);
-  float* ps = qs + dim;
-  long* offs = reinterpret_cast<long*>(lds_raw + wave * per_wave + (static_cast<size_t>(dim) * 4 + kWave * 4 + 7) / 8 * 8);
+  // the block: dim floats of q; per wave 64 weights and 64 value-row offsets; then the waves' shares
+  float* qs = reinterpret_cast<float*>(lds_raw);
+  const size_t q_bytes = (static_cast<size_t>(dim) * 4 + 7) / 8 * 8;
+  float* ps = reinterpret_cast<float*>(lds_raw + q_bytes) + wave * kWave;
+  long* offs = reinterpret_cast<long*>(lds_raw + q_bytes + kRowWaves * kWave * 4) + wave * kWave;
+  float* shares = reinterpret_cast<float*>(lds_raw + q_bytes + kRowWaves * kWave * 12);   // [waves][2 + vdim]
 
   const long n = row / q_heads;
   const int h = static_cast<int>(row % q_heads);
@@ -92,13 +116,13 @@ __global__ __launch_bounds__(256) void gated_attention_rows_kernel(
   const int pos = positions[n];
   int lowest = window > 0 ? max(0, pos - window + 1) : 0;
   if (chunk > 0) lowest = max(lowest, pos / chunk * chunk);
-  for (int i = lane; i < dim; i += kWave) qs[i] = to_float(q[row * dim + i]);
-  wave_sync_lds();
+  for (int i = threadIdx.x; i < dim; i += blockDim.x) qs[i] = to_float(q[row * dim + i]);
+  __syncthreads();
 
-  // with a sink the sums start as if a key of score 0 and no value had been seen
-  float m = sink ? 0.f : -INFINITY, l = sink ? 1.f : 0.f;
+  // with a sink the sums start as if a key of score 0 and no value had been seen (in the first wave's share)
+  float m = sink && wave == 0 ? 0.f : -INFINITY, l = sink && wave == 0 ? 1.f : 0.f;
   float acc[kMaxValueRegs] = {0.f, 0.f, 0.f, 0.f};
-  for (int tile = lowest / kWave; tile * kWave <= pos; ++tile) {
+  for (int tile = lowest / kWave + wave; tile * kWave <= pos; tile += kRowWaves) {
     const int j = tile * kWave + lane;
     const bool valid = j >= lowest && j <= pos;
     float s = -INFINITY;
@@ -110,42 +134,123 @@ __global__ __launch_bounds__(256) void gated_attention_rows_kernel(
       } else {
         const T* kp = k_pages + ((page * kv_heads + kvh) * page_size + j % page_size) * dim;
         float dot = 0.f;
-        for (int i = 0; i < dim; ++i) dot = fmaf(qs[i], to_float(kp[i]), dot);
+        int i = 0;
+        if (VEC) {
+          for (; i + 32 <= dim; i += 32) {       // four loads are asked for before the first is used
+            float kv[4][8];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) load8(kp + i + 8 * u, kv[u]);
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+#pragma unroll
+              for (int e = 0; e < 8; ++e) dot = fmaf(qs[i + 8 * u + e], kv[u][e], dot);
+          }
+          for (; i + 8 <= dim; i += 8) {
+            float kv[8];
+            load8(kp + i, kv);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) dot = fmaf(qs[i + e], kv[e], dot);
+          }
+        }
+        for (; i < dim; ++i) dot = fmaf(qs[i], to_float(kp[i]), dot);
         s = dot * scale;
         if (softcap > 0.f) s = softcap * tanhf(s / softcap);
         value_at = (page * kv_heads + kvh) * vdim * page_size + j % page_size;  // values are [vdim, page_size]
       }
     }
-    const float m_new = fmaxf(m, wave_max(s));
+    const float tile_max = wave_max(s);
+    const float m_new = fmaxf(m, tile_max);
     const float p = valid ? expf(s - m_new) : 0.f;
-    const float correction = expf(m - m_new);
+    const float correction = m_new == m ? 1.f : expf(m - m_new);
     l = l * correction + wave_sum(p);
     m = m_new;
-    ps[lane] = p;
+    ps[lane] = value_at >= 0 || !VEC ? p : 0.f;
     offs[lane] = value_at;
     wave_sync_lds();
 #pragma unroll
     for (int c = 0; c < kMaxValueRegs; ++c) acc[c] *= correction;
-    for (int jj = 0; jj < kWave; ++jj) {
-      const long at = offs[jj];
-      if (at < 0) continue;  // uniform over the wave
-      const float pj = ps[jj];
+    if (VEC) {
+      // a group of eight keys shares a page: its first key that counts tells where the group's values lie
+      long ats[8];
+#pragma unroll
+      for (int g = 0; g < 8; ++g) {
+        long at = -1;
+#pragma unroll
+        for (int e = 7; e >= 0; --e)
+          if (offs[8 * g + e] >= 0) at = offs[8 * g + e] - e;
+        ats[g] = at;
+      }
 #pragma unroll
       for (int c = 0; c < kMaxValueRegs; ++c) {
         const int i = lane + c * kWave;
-        if (i < vdim) acc[c] = fmaf(pj, to_float(v_pages[at + static_cast<long>(i) * page_size]), acc[c]);
+        if (i >= vdim) continue;
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {       // four groups' values are asked for before the first is used
+          float values[4][8];
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            const long at = ats[4 * half + u];
+            if (at >= 0) {
+              load8(v_pages + at + static_cast<long>(i) * page_size, values[u]);
+            } else {
+#pragma unroll
+              for (int e = 0; e < 8; ++e) values[u][e] = 0.f;
+            }
+          }
+#pragma unroll
+          for (int u = 0; u < 4; ++u)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+              const float weight = ps[8 * (4 * half + u) + e];
+              acc[c] += weight != 0.f ? weight * values[u][e] : 0.f;
+            }
+        }
+      }
+    } else {
+      for (int jj = 0; jj < kWave; ++jj) {
+        const long at = offs[jj];
+        if (at < 0) continue;  // uniform over the wave
+        const float pj = ps[jj];
+#pragma unroll
+        for (int c = 0; c < kMaxValueRegs; ++c) {
+          const int i = lane + c * kWave;
+          if (i < vdim) acc[c] = fmaf(pj, to_float(v_pages[at + static_cast<long>(i) * page_size]), acc[c]);
+        }
       }
     }
     wave_sync_lds();
   }
-  float gate = out_scale;
-  if (gates != nullptr) gate = out_scale / (1.f + expf(-to_float(gates[n * gate_stride + gate_at + h])));
+  float* mine = shares + wave * (2 + vdim);
+  if (lane == 0) mine[0] = m, mine[1] = l;
 #pragma unroll
   for (int c = 0; c < kMaxValueRegs; ++c) {
     const int i = lane + c * kWave;
-    if (i < vdim) out[n * out_stride + static_cast<long>(h) * vdim + i] = from_float<T>(acc[c] / l * gate);
+    if (i < vdim) mine[2 + i] = acc[c];
+  }
+  __syncthreads();
+  float highest = -INFINITY;
+  for (int w = 0; w < kRowWaves; ++w) highest = fmaxf(highest, shares[w * (2 + vdim)]);
+  float total = 0.f, factors[kMaxRowWaves];
+#pragma unroll
+  for (int w = 0; w < kMaxRowWaves; ++w) {
+    const float m_w = w < kRowWaves ? shares[w * (2 + vdim)] : -INFINITY;
+    factors[w] = m_w == -INFINITY ? 0.f : expf(m_w - highest);
+    total += w < kRowWaves ? shares[w * (2 + vdim) + 1] * factors[w] : 0.f;
+  }
+  float gate = out_scale;
+  if (gates != nullptr) gate = out_scale / (1.f + expf(-to_float(gates[n * gate_stride + gate_at + h])));
+  for (int i = threadIdx.x; i < vdim; i += blockDim.x) {
+    float sum = 0.f;
+#pragma unroll
+    for (int w = 0; w < kMaxRowWaves; ++w)
+      if (w < kRowWaves) sum += shares[w * (2 + vdim) + 2 + i] * factors[w];
+    out[n * out_stride + static_cast<long>(h) * vdim + i] = from_float<T>(sum / total * gate);
   }
 }
+
+}  // namespace
+
+namespace {
 
 // ---- prompt portions on the matrix cores ----------------------------------------------------------------------------
 // bfloat16, keys 16 DT and values 16 VT wide, pages of a multiple of 16 tokens.  A wave is 16 neighbouring rows of the
@@ -177,10 +282,12 @@ __global__ __launch_bounds__(256) void gated_attention_tiles_kernel(
     int kv_heads, int page_size, long num_pages, float scale, float softcap, int chunk, int window, int sink,
     long out_stride, float out_scale) {
   constexpr int DIM = 32 * DT, VDIM = 16 * VT;
-  const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
-  const int tiles = (tokens - first_row + 15) / 16;
-  const long item = static_cast<long>(blockIdx.x) * (blockDim.x / kWave) + wave;
-  if (item >= static_cast<long>(tiles) * q_heads) return;
+  extern __shared__ float tile_shares[];      // [waves][2 + 4 VT][64]: what the block's waves found over their keys
+  // a block is 16 rows and a head; its waves take the steps of 16 keys in turn
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1), waves = blockDim.x / kWave;
+  // (blocks go to the XCDs in turn: the heads of a tile, which share keys and values, are given to blocks of one XCD)
+  const long item = static_cast<long>(blockIdx.x % kXcds) * (gridDim.x / kXcds) + blockIdx.x / kXcds;
+  if (item >= static_cast<long>((tokens - first_row + 15) / 16) * q_heads) return;
   const int head = static_cast<int>(item % q_heads), tile = static_cast<int>(item / q_heads);
   const int kvh = head / (q_heads / kv_heads);
   const int col = lane & 15, grp = lane >> 4;
@@ -200,7 +307,8 @@ __global__ __launch_bounds__(256) void gated_attention_tiles_kernel(
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) qb[dt] = make_uint4(0u, 0u, 0u, 0u);
   }
-  float m = sink ? 0.f : -INFINITY, l = sink ? 1.f : 0.f;
+  float m = sink && wave == 0 ? 0.f : -INFINITY, l = sink && wave == 0 ? 1.f : 0.f;
+  const float inverse_cap = softcap > 0.f ? 1.f / softcap : 0.f;
   float4_t o[VT];
 #pragma unroll
   for (int vt = 0; vt < VT; ++vt) o[vt] = float4_t{0.f, 0.f, 0.f, 0.f};
@@ -230,10 +338,10 @@ __global__ __launch_bounds__(256) void gated_attention_tiles_kernel(
       for (int vt = 0; vt < VT; ++vt) vs[vt] = load_bf16x4(vp + static_cast<long>(vt) * 16 * page_size);
       return true;
     };
-    const int j_first = lo_run & ~15;
-    there = fetch(j_first, keys, values);
-    for (int j0 = j_first; j0 <= p_last; j0 += 16) {
-      there_next = j0 + 16 <= p_last ? fetch(j0 + 16, keys_next, values_next) : false;
+    const int j_first = (lo_run & ~15) + wave * 16, j_step = waves * 16;
+    if (j_first <= p_last) there = fetch(j_first, keys, values);
+    for (int j0 = j_first; j0 <= p_last; j0 += j_step) {
+      there_next = j0 + j_step <= p_last ? fetch(j0 + j_step, keys_next, values_next) : false;
       if (there) {
         float4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -246,18 +354,21 @@ __global__ __launch_bounds__(256) void gated_attention_tiles_kernel(
         for (int i = 0; i < 4; ++i) {
           const int j = j0 + grp * 4 + i;
           float v = acc[i] * scale;
-          if (softcap > 0.f) v = softcap * tanhf(v / softcap);
+          if (softcap > 0.f) {      // tanh(x) = 1 - 2 / (exp(2 x) + 1), with the hardware's exponential and reciprocal
+            const float e = __expf(2.f * fabsf(v) * inverse_cap);
+            v = copysignf(softcap * (1.f - 2.f * __frcp_rn(e + 1.f)), v);
+          }
           s[i] = (in_run && j >= my_lowest && j <= my_pos) ? v : -INFINITY;
           highest = fmaxf(highest, s[i]);
         }
         highest = fmaxf(highest, __shfl_xor(highest, 16, kWave));
         highest = fmaxf(highest, __shfl_xor(highest, 32, kWave));
         const float m_new = fmaxf(m, highest);
-        const float correction = m_new == m ? 1.f : expf(m - m_new);
+        const float correction = m_new == m ? 1.f : __expf(m - m_new);
         float p[4], added = 0.f;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          p[i] = s[i] == -INFINITY ? 0.f : expf(s[i] - m_new);
+          p[i] = s[i] == -INFINITY ? 0.f : __expf(s[i] - m_new);
           added += p[i];
         }
         added += __shfl_xor(added, 16, kWave);
@@ -295,6 +406,34 @@ __global__ __launch_bounds__(256) void gated_attention_tiles_kernel(
     }
     row = run_end;
   }
+  if (waves > 1) {      // the waves' shares meet in LDS and the first wave adds them in the order of the waves
+    float* mine = tile_shares + static_cast<size_t>(wave) * (2 + 4 * VT) * kWave + lane;
+    mine[0] = m;
+    mine[kWave] = l;
+#pragma unroll
+    for (int vt = 0; vt < VT; ++vt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) mine[(2 + 4 * vt + i) * kWave] = o[vt][i];
+    __syncthreads();
+    if (wave != 0) return;
+    float highest = m;
+    for (int w = 1; w < waves; ++w) highest = fmaxf(highest, tile_shares[static_cast<size_t>(w) * (2 + 4 * VT) * kWave + lane]);
+    const float own = m == -INFINITY ? 0.f : expf(m - highest);
+    l *= own;
+#pragma unroll
+    for (int vt = 0; vt < VT; ++vt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[vt][i] *= own;
+    for (int w = 1; w < waves; ++w) {
+      const float* other = tile_shares + static_cast<size_t>(w) * (2 + 4 * VT) * kWave + lane;
+      const float factor = other[0] == -INFINITY ? 0.f : expf(other[0] - highest);
+      l += other[kWave] * factor;
+#pragma unroll
+      for (int vt = 0; vt < VT; ++vt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[vt][i] += other[(2 + 4 * vt + i) * kWave] * factor;
+    }
+  }
   if (!have) return;
   float gate = out_scale;
   if (gates != nullptr) gate = out_scale / (1.f + expf(-to_float(gates[static_cast<long>(my_row) * gate_stride + gate_at + head])));
@@ -324,9 +463,11 @@ int akv_gated_attention_tiles(const void* q, const void* k_pages, const void* v_
   if (tokens <= first_row) return 0;
   if (page_size % 16 != 0 || q_heads % kv_heads != 0) return -2;
   const long items = static_cast<long>((tokens - first_row + 15) / 16) * q_heads;
-  const unsigned grid = static_cast<unsigned>((items + 3) / 4);
+  const unsigned grid = static_cast<unsigned>((items + kXcds - 1) / kXcds * kXcds);
+  const int waves = vdim > 128 ? 2 : 4;       // (their shares must fit into 64 KB of LDS)
+  const size_t lds = static_cast<size_t>(waves) * (2 + vdim / 4) * kWave * 4;
 #define AKV_TILES(DT, VT)                                                                                              \
-  gated_attention_tiles_kernel<DT, VT><<<grid, 256, 0, stream>>>(                                                      \
+  gated_attention_tiles_kernel<DT, VT><<<grid, waves * kWave, lds, stream>>>(                                                    \
       static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_pages), static_cast<const bf16_t*>(v_pages),         \
       static_cast<const bf16_t*>(gates), gate_stride, gate_at, seq_of_token, q_start, positions, block_table, table_rows, \
       table_width, static_cast<bf16_t*>(out), first_row, tokens, q_heads, kv_heads, page_size, num_pages, scale, softcap, \
@@ -368,19 +509,31 @@ int akv_gated_attention_rows(const void* q, const void* k_pages, const void* v_p
                              int gate_at, const int* seq_of_token, const int* positions, const int* block_table,
                              const int* table_rows, int table_width, void* out, int dtype, long tokens, int q_heads,
                              int kv_heads, int dim, int vdim, int page_size, long num_pages, float scale, float softcap,
-                             int chunk, int window, int sink, long out_stride, float out_scale, hipStream_t stream) {
+                             int chunk, int window, int sink, long out_stride, float out_scale, int row_waves,
+                             hipStream_t stream) {
   if (tokens <= 0) return 0;
+  const int kRowWaves = row_waves;
+  if (row_waves < 1 || row_waves > kMaxRowWaves) return -2;
   if (vdim > kMaxValueRegs * kWave || dim <= 0 || q_heads % kv_heads != 0) return -2;
   const long rows = tokens * q_heads;
-  const size_t per_wave = (static_cast<size_t>(dim) * 4 + kWave * 4 + kWave * 8 + 7) / 8 * 8;
-  const size_t lds = 4 * per_wave;
+  const size_t q_bytes = (static_cast<size_t>(dim) * 4 + 7) / 8 * 8;
+  const size_t lds = q_bytes + kRowWaves * kWave * 12 + static_cast<size_t>(kRowWaves) * (2 + vdim) * 4;
   if (lds > 64 * 1024) return -2;
-  AKV_DISPATCH(dtype, T,
-               gated_attention_rows_kernel<T><<<static_cast<unsigned>((rows + 3) / 4), 256, lds, stream>>>(
-                   static_cast<const T*>(q), static_cast<const T*>(k_pages), static_cast<const T*>(v_pages),
-                   static_cast<const T*>(gates), gate_stride, gate_at, seq_of_token, positions, block_table, table_rows,
-                   table_width, static_cast<T*>(out), tokens, q_heads, kv_heads, dim, vdim, page_size, num_pages, scale,
-                   softcap, chunk, window, sink, out_stride, out_scale));
+  const size_t element = dtype == kBF16 ? 2 : 4;
+  // 16-byte loads: key rows and groups of eight neighbouring keys' values must be aligned
+  const bool vec = (dim * element) % 16 == 0 && page_size % 8 == 0 && (8 * element) % 16 == 0 &&
+                   (static_cast<size_t>(page_size) * element) % 16 == 0 && reinterpret_cast<uintptr_t>(k_pages) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(v_pages) % 16 == 0;
+#define AKV_ROWS(VEC)                                                                                                   \
+  AKV_DISPATCH(dtype, T,                                                                                                \
+               gated_attention_rows_kernel<T, VEC><<<static_cast<unsigned>((rows + kXcds - 1) / kXcds * kXcds), kRowWaves * kWave, lds, stream>>>(    \
+                   static_cast<const T*>(q), static_cast<const T*>(k_pages), static_cast<const T*>(v_pages),            \
+                   static_cast<const T*>(gates), gate_stride, gate_at, seq_of_token, positions, block_table, table_rows, \
+                   table_width, static_cast<T*>(out), tokens, q_heads, kv_heads, dim, vdim, page_size, num_pages, scale, \
+                   softcap, chunk, window, sink, out_stride, out_scale))
+  if (vec) AKV_ROWS(true);
+  else AKV_ROWS(false);
+#undef AKV_ROWS
   return AKV_LAUNCH_STATUS();
 }
 }

@@ -469,10 +469,15 @@ class PartsKernels:
                 _ptr_at(out, out_at), singles, tokens, q_heads, kv_heads, dim, vdim, page_size, _long(num_pages), *tail),
                 "gated_attention on the matrix cores")
         if singles:
+            # waves that share a token's head: by the most keys a row can see (a bound that a recorded step keeps), fewer
+            # where the rows alone fill the device
+            span = min(x for x in (chunk, window, ctx.max_seq_len) if x is not None)
+            row_waves = max(1, min(16 if singles * q_heads <= 4096 else 4, span // 128))
             self._check(self._parts().akv_gated_attention_rows(
                 _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(gates), _long(gate_stride), gate_at, _ptr(ctx.seq_of_token),
                 _ptr(ctx.positions), _ptr(meta.block_table), _ptr(meta.rows), meta.width, _ptr_at(out, out_at),
-                self._code_of(q), _long(singles), q_heads, kv_heads, dim, vdim, page_size, _long(num_pages), *tail), "gated_attention")
+                self._code_of(q), _long(singles), q_heads, kv_heads, dim, vdim, page_size, _long(num_pages), *tail[:-1], row_waves,
+                tail[-1]), "gated_attention")
 
     # ---- mixers with a state of fixed size -----------------------------------------------------------------------------
     def check_retention_sizes(self, heads: int, dim: int, vdim: int) -> None:

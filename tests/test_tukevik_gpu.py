@@ -167,13 +167,13 @@ def _ctx(lengths_before, counts, device=DEVICE):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("heads,kv_heads,dim,vdim,chunk,page", [(4, 2, 16, 24, 11, 4), (3, 1, 40, 8, 64, 16), (8, 8, 64, 64, 7, 8),
                                                                (2, 1, 128, 256, 300, 16), (8, 2, 64, 32, 20, 16),
-                                                               (4, 4, 32, 128, 48, 32)])
+                                                               (4, 4, 32, 128, 48, 32), (1, 1, 64, 64, 5000, 16)])
 def test_attention_kernel_alone(hip, dtype, heads, kv_heads, dim, vdim, chunk, page):
     """Two requests in two portions each, through the unit norm with its cache write and the attention, against the plain
     attention of the whole sequences.  Scores are made sharp, and one key a request - the first of a chunk - is made to
     stand out for every later query: it counts up to its chunk's last position and not beyond."""
     torch.manual_seed(heads * 100 + dim)
-    lengths, eps, scale, softcap = (75, 2 * chunk + 3 if chunk < 100 else 330), 1e-6, 1.2, 9.0
+    lengths, eps, scale, softcap = (75, 2 * chunk + 3 if chunk < 100 else 330 if chunk < 1000 else 2100), 1e-6, 1.2, 9.0
     m = dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim, mask=dict(size=chunk), scale=scale, softcap=softcap)
     width = heads * dim + kv_heads * (dim + vdim) + heads
     rows = [torch.randn(n, width) for n in lengths]
@@ -190,8 +190,9 @@ def test_attention_kernel_alone(hip, dtype, heads, kv_heads, dim, vdim, chunk, p
         for i in range((n + page - 1) // page):
             table[r, i] = order.pop()
     got = [torch.zeros(n, heads * vdim) for n in lengths]
-    for step, befores in enumerate([(0, 0), (41, 5)]):
-        counts = [41, 5] if step == 0 else [lengths[0] - 41, lengths[1] - 5]
+    # two portions each, then the last token of each alone (sixteen waves share a row whose request is long)
+    for step, befores in enumerate([(0, 0), (41, 5), (lengths[0] - 1, lengths[1] - 1)]):
+        counts = [[41, 5], [lengths[0] - 42, lengths[1] - 6], [1, 1]][step]
         ctx = _ctx(befores, counts)
         projected = torch.cat([rows[r][b:b + c] for r, (b, c) in enumerate(zip(befores, counts))]).to(dtype).to(DEVICE)
         slot_map = torch.tensor([int(table[r, p // page]) * page + p % page for r, (b, c) in enumerate(zip(befores, counts))

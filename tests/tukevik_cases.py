@@ -199,12 +199,12 @@ def case_first_tokens(engine, case):
     check(engine, sub, [([("x", 1), ("y", 2), ("z", 1)], ["x"]), ([("y", 1), ("z", 1)], ["y", "z"])])
 
 
-def case_long_decoding(engine, case):
+def case_long_decoding(engine, case, tokens: int = 230):
     """Every chunk's edge passes under decoded tokens many times, the pages of chunks that were left are given back and
     taken again while the request lives, and the states carry two hundred steps."""
-    ids = random_ids(case["raw"]["vocab"], 230, seed=77)
+    ids = random_ids(case["raw"]["vocab"], tokens, seed=77)
     sub = dict(case, requests={"long": ids}, expected={"long": plain_logits(case["folder"], ids)})
-    check(engine, sub, schedules.last_one_by_one({"long": ids}, 220))
+    check(engine, sub, schedules.last_one_by_one({"long": ids}, tokens - 10))
 
 
 def case_greedy_generation(engine, case):
