@@ -274,7 +274,7 @@ __device__ __forceinline__ uint4 load_bf16x8(const bf16_t* p) { return *reinterp
 
 // DT: key width / 32 (the first product runs in steps of 32 dimensions), VT: value width / 16.
 template <int DT, int VT>
-__global__ __launch_bounds__(256) void gated_attention_tiles_kernel(
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((DT + VT <= 12 ? 3 : 2), 4))) void gated_attention_tiles_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     const bf16_t* __restrict__ gates, long gate_stride, int gate_at, const int* __restrict__ seq_of_token,
     const int* __restrict__ q_start, const int* __restrict__ positions, const int* __restrict__ block_table,
@@ -285,10 +285,13 @@ __global__ __launch_bounds__(256) void gated_attention_tiles_kernel(
   extern __shared__ float tile_shares[];      // [waves][2 + 4 VT][64]: what the block's waves found over their keys
   // a block is 16 rows and a head; its waves take the steps of 16 keys in turn
   const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1), waves = blockDim.x / kWave;
-  // (blocks go to the XCDs in turn: the heads of a tile, which share keys and values, are given to blocks of one XCD)
-  const long item = static_cast<long>(blockIdx.x % kXcds) * (gridDim.x / kXcds) + blockIdx.x / kXcds;
-  if (item >= static_cast<long>((tokens - first_row + 15) / 16) * q_heads) return;
-  const int head = static_cast<int>(item % q_heads), tile = static_cast<int>(item / q_heads);
+  // blocks go to the XCDs in turn: the heads of a tile, which share keys and values, are given to blocks of one XCD, the
+  // tiles to the XCDs in turn, and the tiles with the most keys before them - the last of a portion - start first
+  const int tiles = (tokens - first_row + 15) / 16;
+  const int slot = blockIdx.x / kXcds;
+  const int head = slot % q_heads, turned = slot / q_heads * kXcds + blockIdx.x % kXcds;
+  if (turned >= tiles) return;
+  const int tile = tiles - 1 - turned;
   const int kvh = head / (q_heads / kv_heads);
   const int col = lane & 15, grp = lane >> 4;
   const int row0 = first_row + tile * 16, row_end = min(row0 + 16, tokens);
@@ -463,7 +466,7 @@ int akv_gated_attention_tiles(const void* q, const void* k_pages, const void* v_
   if (tokens <= first_row) return 0;
   if (page_size % 16 != 0 || q_heads % kv_heads != 0) return -2;
   const long items = static_cast<long>((tokens - first_row + 15) / 16) * q_heads;
-  const unsigned grid = static_cast<unsigned>((items + kXcds - 1) / kXcds * kXcds);
+  const unsigned grid = static_cast<unsigned>(((tokens - first_row + 15) / 16 + kXcds - 1) / kXcds * kXcds * q_heads);
   const int waves = vdim > 128 ? 2 : 4;       // (their shares must fit into 64 KB of LDS)
   const size_t lds = static_cast<size_t>(waves) * (2 + vdim / 4) * kWave * 4;
 #define AKV_TILES(DT, VT)                                                                                              \
