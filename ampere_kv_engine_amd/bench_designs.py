@@ -59,15 +59,15 @@ TUKEVIK_SIZES = {
 def tukevik_config(size: dict, layers: int) -> dict:
     parallel = dict(
         left=dict(heads=size["heads"], kv_heads=size["kv_heads"], dim=size["dim"], vdim=size["vdim"], mask=dict(size=size["chunk"]),
-                  scale=size["dim"] ** -0.5, softcap=30.0), left_scale=0.8,
-        right=dict(heads=size["r_heads"], dim=size["r_dim"], vdim=size["r_vdim"], rot=dict(base=1e6, dims=size["r_dim"]),
-                   decay=[1.0 - 2.0 ** -(5 + h % 6) for h in range(size["r_heads"])]), right_scale=1.1)
+                  scale=size["dim"] ** -0.5, softcap=50.0), left_scale=0.7,
+        right=dict(heads=size["r_heads"], dim=size["r_dim"], vdim=size["r_vdim"], rot=dict(base=1e4, dims=size["r_dim"]),
+                   decay=[1.0 - 2.0 ** -(5 + h % 6) for h in range(size["r_heads"])]), right_scale=1.2)
     recurrent = dict(width=size["recurrent"], blocks=size["blocks"], conv=size["conv"])
     dense = dict(kind="dense", ff=size["dense"])
     routed = dict(kind="moe", expert=dict(ff=size["ff"]), router=dict(experts=size["experts"], top=size["top"]),
                   shared=dict(ff=size["shared"]))
     pattern = [("parallel", parallel, dense), ("rglru", recurrent, routed), ("rglru", recurrent, dense), ("parallel", parallel, routed)]
-    return dict(architecture="Tukevik", vocab=size["vocab"], width=size["width"], norm=dict(eps=1e-6), residual_mult=0.5,
+    return dict(architecture="Tukevik", vocab=size["vocab"], width=size["width"], norm=dict(eps=1e-6), residual_mult=0.6,
                 layers=[dict(type=kind, mixer=mixer, mlp=mlp) for kind, mixer, mlp in (pattern[i % 4] for i in range(layers))])
 
 

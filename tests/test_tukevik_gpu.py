@@ -310,7 +310,8 @@ def test_recurrent_unit_kernels_alone(hip, dtype, width, blocks, taps):
         assert error < (2e-5 if dtype == torch.float32 else 0.04), f"request {r}: {error:.2e}"
 
 
-@pytest.mark.parametrize("experts,top,ff,shared", [(6, 3, 20, 28), (4, 1, 16, 0), (2, 2, 8, 8), (70, 5, 4, 12), (1, 1, 8, 0)])
+@pytest.mark.parametrize("experts,top,ff,shared", [(6, 3, 20, 28), (4, 1, 16, 0), (2, 2, 8, 8), (70, 5, 4, 12), (1, 1, 8, 0),
+                                                   (5, 2, 24, 40)])
 def test_routing_and_the_experts_activation(hip, experts, top, ff, shared):
     torch.manual_seed(experts)
     tokens = 37

@@ -50,10 +50,10 @@ TUKEVIK_B = dict(
     ])
 # Sizes in multiples of 64 - what a served model has - with a chunk longer than most requests and one of three pages.
 TUKEVIK_C = dict(
-    architecture="Tukevik", vocab=300, width=128, norm=dict(eps=1e-5), residual_mult=0.5,
+    architecture="Tukevik", vocab=300, width=128, norm=dict(eps=1e-5), residual_mult=0.6,
     layers=[
-        dict(type="parallel", mlp=DENSE(256),
-             mixer=PARALLEL(LEFT(8, 2, 64, 64, 48, 0.7, 30.0), RIGHT(2, 64, 64, [0.984375, 0.9990234375], 32, 1e4), 0.8, 1.1)),
+        dict(type="parallel", mlp=DENSE(192),
+             mixer=PARALLEL(LEFT(8, 2, 64, 64, 48, 0.7, 25.0), RIGHT(2, 64, 64, [0.96875, 0.998], 32, 1e4), 0.9, 1.2)),
         dict(type="rglru", mixer=RGLRU(256, 4, 4), mlp=MOE(8, 2, 64, 64)),
         dict(type="parallel", mlp=MOE(4, 2, 128, None),
              mixer=PARALLEL(LEFT(4, 4, 128, 64, 200, 0.5, 20.0), RIGHT(2, 128, 64, [0.99, 0.999], 128, 1e4), 1.0, 1.0)),
