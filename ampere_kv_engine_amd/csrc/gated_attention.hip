@@ -85,11 +85,13 @@ __device__ __forceinline__ void load8(const float* p, float (&v)[8]) {
   v[0] = a.x, v[1] = a.y, v[2] = a.z, v[3] = a.w, v[4] = b.x, v[5] = b.y, v[6] = b.z, v[7] = b.w;
 }
 
-// A block is a (token, query head); its waves (1 to 16, the caller's choice) take the row's key tiles in turn and their shares - maximum, sum of
-// weights, weighted values - meet in LDS in the order of the waves.  Inside a tile a lane scores one key (VEC: its
-// dimensions eight at a time) and then owns value dimensions, for which it reads eight neighbouring keys' values at a
-// time (the value pages lie [vdim, page]).  VEC needs key rows and groups of eight values that are 16-byte aligned.
-template <typename T, bool VEC>
+// A block is a token and G query heads that read the same key head (G = 1: a single head); its waves (1 to 16, the
+// caller's choice) take the row's tiles of 64 keys in turn and their shares - maximum, sum of weights, weighted values,
+// per head - meet in LDS in the order of the waves.  Inside a tile a lane scores one key for all G heads from one read of
+// it (VEC: its dimensions eight at a time) and then owns value dimensions, for which it reads eight neighbouring keys'
+// values at a time (the value pages lie [vdim, page]) - once for the G heads.  VEC needs key rows and groups of eight
+// values that are 16-byte aligned.
+template <typename T, bool VEC, int G>
 __global__ __launch_bounds__(kMaxRowWaves * kWave) void gated_attention_rows_kernel(
     const T* __restrict__ q, const T* __restrict__ k_pages, const T* __restrict__ v_pages, const T* __restrict__ gates,
     long gate_stride, int gate_at, const int* __restrict__ seq_of_token, const int* __restrict__ positions,
@@ -98,153 +100,181 @@ __global__ __launch_bounds__(kMaxRowWaves * kWave) void gated_attention_rows_ker
     int chunk, int window, int sink, long out_stride, float out_scale) {
   extern __shared__ unsigned char lds_raw[];
   const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1), kRowWaves = blockDim.x / kWave;
-  // blocks go to the XCDs in turn: neighbouring rows - the query heads of one key head, which read the same keys and
-  // values - are given to blocks of one XCD, whose L2 then fetches those once
+  // blocks go to the XCDs in turn: neighbouring rows - which read the same or neighbouring keys and values - are given to
+  // blocks of one XCD
   const long row = static_cast<long>(blockIdx.x % kXcds) * (gridDim.x / kXcds) + blockIdx.x / kXcds;
-  if (row >= tokens * q_heads) return;
-  // the block: dim floats of q; per wave 64 weights and 64 value-row offsets; then the waves' shares
+  const int bundles = q_heads / G;           // rows of a token
+  if (row >= tokens * bundles) return;
+  // the block: G x dim floats of q; per wave G x 64 weights and 64 value-row offsets; then the waves' shares
   float* qs = reinterpret_cast<float*>(lds_raw);
-  const size_t q_bytes = (static_cast<size_t>(dim) * 4 + 7) / 8 * 8;
-  float* ps = reinterpret_cast<float*>(lds_raw + q_bytes) + wave * kWave;
-  long* offs = reinterpret_cast<long*>(lds_raw + q_bytes + kRowWaves * kWave * 4) + wave * kWave;
-  float* shares = reinterpret_cast<float*>(lds_raw + q_bytes + kRowWaves * kWave * 12);   // [waves][2 + vdim]
+  const size_t q_bytes = (static_cast<size_t>(G) * dim * 4 + 7) / 8 * 8;
+  float* ps = reinterpret_cast<float*>(lds_raw + q_bytes) + wave * G * kWave;
+  long* offs = reinterpret_cast<long*>(lds_raw + q_bytes + static_cast<size_t>(kRowWaves) * G * kWave * 4) + wave * kWave;
+  float* shares = reinterpret_cast<float*>(lds_raw + q_bytes + static_cast<size_t>(kRowWaves) * kWave * (G * 4 + 8));
 
-  const long n = row / q_heads;
-  const int h = static_cast<int>(row % q_heads);
-  const int kvh = h / (q_heads / kv_heads);
+  const long n = row / bundles;
+  const int h0 = static_cast<int>(row % bundles) * G;
+  const int kvh = h0 / (q_heads / kv_heads);
   const int r = table_rows != nullptr ? table_rows[seq_of_token[n]] : seq_of_token[n];
   const int pos = positions[n];
   int lowest = window > 0 ? max(0, pos - window + 1) : 0;
   if (chunk > 0) lowest = max(lowest, pos / chunk * chunk);
-  for (int i = threadIdx.x; i < dim; i += blockDim.x) qs[i] = to_float(q[row * dim + i]);
+  for (int i = threadIdx.x; i < G * dim; i += blockDim.x) qs[i] = to_float(q[(n * q_heads + h0) * dim + i]);
   __syncthreads();
 
   // with a sink the sums start as if a key of score 0 and no value had been seen (in the first wave's share)
-  float m = sink && wave == 0 ? 0.f : -INFINITY, l = sink && wave == 0 ? 1.f : 0.f;
-  float acc[kMaxValueRegs] = {0.f, 0.f, 0.f, 0.f};
+  float m[G], l[G], acc[G][kMaxValueRegs];
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    m[g] = sink && wave == 0 ? 0.f : -INFINITY;
+    l[g] = sink && wave == 0 ? 1.f : 0.f;
+#pragma unroll
+    for (int c = 0; c < kMaxValueRegs; ++c) acc[g][c] = 0.f;
+  }
   for (int tile = lowest / kWave + wave; tile * kWave <= pos; tile += kRowWaves) {
     const int j = tile * kWave + lane;
     const bool valid = j >= lowest && j <= pos;
-    float s = -INFINITY;
+    float s[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) s[g] = -INFINITY;
     long value_at = -1;
     if (valid) {
       const long page = block_table[static_cast<long>(r) * table_width + j / page_size];
       if (page < 0 || page >= num_pages) {
-        s = __uint_as_float(0x7fc00000u);  // a page that is not the request's: poison, never read
+#pragma unroll
+        for (int g = 0; g < G; ++g) s[g] = __uint_as_float(0x7fc00000u);  // a page that is not the request's: poison
       } else {
         const T* kp = k_pages + ((page * kv_heads + kvh) * page_size + j % page_size) * dim;
-        float dot = 0.f;
+        float dot[G];
+#pragma unroll
+        for (int g = 0; g < G; ++g) dot[g] = 0.f;
         int i = 0;
         if (VEC) {
-          for (; i + 32 <= dim; i += 32) {       // four loads are asked for before the first is used
-            float kv[4][8];
+          for (; i + 16 <= dim; i += 16) {       // two loads are asked for before the first is used
+            float kv[2][8];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) load8(kp + i + 8 * u, kv[u]);
+            for (int u = 0; u < 2; ++u) load8(kp + i + 8 * u, kv[u]);
 #pragma unroll
-            for (int u = 0; u < 4; ++u)
+            for (int u = 0; u < 2; ++u)
 #pragma unroll
-              for (int e = 0; e < 8; ++e) dot = fmaf(qs[i + 8 * u + e], kv[u][e], dot);
+              for (int e = 0; e < 8; ++e)
+#pragma unroll
+                for (int g = 0; g < G; ++g) dot[g] = fmaf(qs[g * dim + i + 8 * u + e], kv[u][e], dot[g]);
           }
           for (; i + 8 <= dim; i += 8) {
             float kv[8];
             load8(kp + i, kv);
 #pragma unroll
-            for (int e = 0; e < 8; ++e) dot = fmaf(qs[i + e], kv[e], dot);
+            for (int e = 0; e < 8; ++e)
+#pragma unroll
+              for (int g = 0; g < G; ++g) dot[g] = fmaf(qs[g * dim + i + e], kv[e], dot[g]);
           }
         }
-        for (; i < dim; ++i) dot = fmaf(qs[i], to_float(kp[i]), dot);
-        s = dot * scale;
-        if (softcap > 0.f) s = softcap * tanhf(s / softcap);
+        for (; i < dim; ++i) {
+          const float kv = to_float(kp[i]);
+#pragma unroll
+          for (int g = 0; g < G; ++g) dot[g] = fmaf(qs[g * dim + i], kv, dot[g]);
+        }
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+          s[g] = dot[g] * scale;
+          if (softcap > 0.f) s[g] = softcap * tanhf(s[g] / softcap);
+        }
         value_at = (page * kv_heads + kvh) * vdim * page_size + j % page_size;  // values are [vdim, page_size]
       }
     }
-    const float tile_max = wave_max(s);
-    const float m_new = fmaxf(m, tile_max);
-    const float p = valid ? expf(s - m_new) : 0.f;
-    const float correction = m_new == m ? 1.f : expf(m - m_new);
-    l = l * correction + wave_sum(p);
-    m = m_new;
-    ps[lane] = value_at >= 0 || !VEC ? p : 0.f;
+    float correction[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      const float m_new = fmaxf(m[g], wave_max(s[g]));
+      const float p = valid ? expf(s[g] - m_new) : 0.f;
+      correction[g] = m_new == m[g] ? 1.f : expf(m[g] - m_new);
+      l[g] = l[g] * correction[g] + wave_sum(p);
+      m[g] = m_new;
+      ps[g * kWave + lane] = value_at >= 0 || !VEC ? p : 0.f;
+    }
     offs[lane] = value_at;
     wave_sync_lds();
 #pragma unroll
-    for (int c = 0; c < kMaxValueRegs; ++c) acc[c] *= correction;
+    for (int g = 0; g < G; ++g)
+#pragma unroll
+      for (int c = 0; c < kMaxValueRegs; ++c) acc[g][c] *= correction[g];
     if (VEC) {
       // a group of eight keys shares a page: its first key that counts tells where the group's values lie
-      long ats[8];
-#pragma unroll
-      for (int g = 0; g < 8; ++g) {
+#pragma unroll 2
+      for (int k = 0; k < 8; ++k) {
         long at = -1;
 #pragma unroll
         for (int e = 7; e >= 0; --e)
-          if (offs[8 * g + e] >= 0) at = offs[8 * g + e] - e;
-        ats[g] = at;
-      }
+          if (offs[8 * k + e] >= 0) at = offs[8 * k + e] - e;
+        if (at < 0) continue;  // uniform over the wave
+        float weights[G][8];
 #pragma unroll
-      for (int c = 0; c < kMaxValueRegs; ++c) {
-        const int i = lane + c * kWave;
-        if (i >= vdim) continue;
+        for (int g = 0; g < G; ++g)
 #pragma unroll
-        for (int half = 0; half < 2; ++half) {       // four groups' values are asked for before the first is used
-          float values[4][8];
+          for (int e = 0; e < 8; ++e) weights[g][e] = ps[g * kWave + 8 * k + e];
 #pragma unroll
-          for (int u = 0; u < 4; ++u) {
-            const long at = ats[4 * half + u];
-            if (at >= 0) {
-              load8(v_pages + at + static_cast<long>(i) * page_size, values[u]);
-            } else {
+        for (int c = 0; c < kMaxValueRegs; ++c) {
+          const int i = lane + c * kWave;
+          if (i < vdim) {
+            float values[8];
+            load8(v_pages + at + static_cast<long>(i) * page_size, values);
 #pragma unroll
-              for (int e = 0; e < 8; ++e) values[u][e] = 0.f;
-            }
+            for (int e = 0; e < 8; ++e)
+#pragma unroll
+              for (int g = 0; g < G; ++g) acc[g][c] += weights[g][e] != 0.f ? weights[g][e] * values[e] : 0.f;
           }
-#pragma unroll
-          for (int u = 0; u < 4; ++u)
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-              const float weight = ps[8 * (4 * half + u) + e];
-              acc[c] += weight != 0.f ? weight * values[u][e] : 0.f;
-            }
         }
       }
     } else {
       for (int jj = 0; jj < kWave; ++jj) {
         const long at = offs[jj];
         if (at < 0) continue;  // uniform over the wave
-        const float pj = ps[jj];
 #pragma unroll
         for (int c = 0; c < kMaxValueRegs; ++c) {
           const int i = lane + c * kWave;
-          if (i < vdim) acc[c] = fmaf(pj, to_float(v_pages[at + static_cast<long>(i) * page_size]), acc[c]);
+          if (i < vdim) {
+            const float value = to_float(v_pages[at + static_cast<long>(i) * page_size]);
+#pragma unroll
+            for (int g = 0; g < G; ++g) acc[g][c] = fmaf(ps[g * kWave + jj], value, acc[g][c]);
+          }
         }
       }
     }
     wave_sync_lds();
   }
-  float* mine = shares + wave * (2 + vdim);
-  if (lane == 0) mine[0] = m, mine[1] = l;
+  const int share = 2 + vdim;
 #pragma unroll
-  for (int c = 0; c < kMaxValueRegs; ++c) {
-    const int i = lane + c * kWave;
-    if (i < vdim) mine[2 + i] = acc[c];
+  for (int g = 0; g < G; ++g) {
+    float* mine = shares + static_cast<size_t>(wave * G + g) * share;
+    if (lane == 0) mine[0] = m[g], mine[1] = l[g];
+#pragma unroll
+    for (int c = 0; c < kMaxValueRegs; ++c) {
+      const int i = lane + c * kWave;
+      if (i < vdim) mine[2 + i] = acc[g][c];
+    }
   }
   __syncthreads();
-  float highest = -INFINITY;
-  for (int w = 0; w < kRowWaves; ++w) highest = fmaxf(highest, shares[w * (2 + vdim)]);
-  float total = 0.f, factors[kMaxRowWaves];
+  for (int g = 0; g < G; ++g) {
+    float highest = -INFINITY;
+    for (int w = 0; w < kRowWaves; ++w) highest = fmaxf(highest, shares[static_cast<size_t>(w * G + g) * share]);
+    float total = 0.f, factors[kMaxRowWaves];
 #pragma unroll
-  for (int w = 0; w < kMaxRowWaves; ++w) {
-    const float m_w = w < kRowWaves ? shares[w * (2 + vdim)] : -INFINITY;
-    factors[w] = m_w == -INFINITY ? 0.f : expf(m_w - highest);
-    total += w < kRowWaves ? shares[w * (2 + vdim) + 1] * factors[w] : 0.f;
-  }
-  float gate = out_scale;
-  if (gates != nullptr) gate = out_scale / (1.f + expf(-to_float(gates[n * gate_stride + gate_at + h])));
-  for (int i = threadIdx.x; i < vdim; i += blockDim.x) {
-    float sum = 0.f;
+    for (int w = 0; w < kMaxRowWaves; ++w) {
+      const float m_w = w < kRowWaves ? shares[static_cast<size_t>(w * G + g) * share] : -INFINITY;
+      factors[w] = m_w == -INFINITY ? 0.f : expf(m_w - highest);
+      total += w < kRowWaves ? shares[static_cast<size_t>(w * G + g) * share + 1] * factors[w] : 0.f;
+    }
+    const int h = h0 + g;
+    float gate = out_scale;
+    if (gates != nullptr) gate = out_scale / (1.f + expf(-to_float(gates[n * gate_stride + gate_at + h])));
+    for (int i = threadIdx.x; i < vdim; i += blockDim.x) {
+      float sum = 0.f;
 #pragma unroll
-    for (int w = 0; w < kMaxRowWaves; ++w)
-      if (w < kRowWaves) sum += shares[w * (2 + vdim) + 2 + i] * factors[w];
-    out[n * out_stride + static_cast<long>(h) * vdim + i] = from_float<T>(sum / total * gate);
+      for (int w = 0; w < kMaxRowWaves; ++w)
+        if (w < kRowWaves) sum += shares[static_cast<size_t>(w * G + g) * share + 2 + i] * factors[w];
+      out[n * out_stride + static_cast<long>(h) * vdim + i] = from_float<T>(sum / total * gate);
+    }
   }
 }
 
@@ -518,24 +548,42 @@ int akv_gated_attention_rows(const void* q, const void* k_pages, const void* v_p
   const int kRowWaves = row_waves;
   if (row_waves < 1 || row_waves > kMaxRowWaves) return -2;
   if (vdim > kMaxValueRegs * kWave || dim <= 0 || q_heads % kv_heads != 0) return -2;
-  const long rows = tokens * q_heads;
-  const size_t q_bytes = (static_cast<size_t>(dim) * 4 + 7) / 8 * 8;
-  const size_t lds = q_bytes + kRowWaves * kWave * 12 + static_cast<size_t>(kRowWaves) * (2 + vdim) * 4;
+  // A block a head.  (The kernel can take 2 or 4 query heads of a key head in one block, reading keys and values once
+  // for them; with a quarter of the blocks at its register count that was slower at 8 requests of 2,048 keys, 16 query
+  // and 4 key heads - 66 us against 39 - and is not chosen.)
+  int bundle = 1;
+  int waves = kRowWaves;
+  auto lds_of = [&](int g, int w) {
+    return (static_cast<size_t>(g) * dim * 4 + 7) / 8 * 8 + static_cast<size_t>(w) * kWave * (g * 4 + 8) +
+           static_cast<size_t>(w) * g * (2 + vdim) * 4;
+  };
+  while (lds_of(bundle, waves) > 64 * 1024 && waves > 1) waves /= 2;
+  while (lds_of(bundle, waves) > 64 * 1024 && bundle > 1) bundle /= 2;
+  const size_t lds = lds_of(bundle, waves);
   if (lds > 64 * 1024) return -2;
+  const long rows = tokens * (q_heads / bundle);
   const size_t element = dtype == kBF16 ? 2 : 4;
   // 16-byte loads: key rows and groups of eight neighbouring keys' values must be aligned
-  const bool vec = (dim * element) % 16 == 0 && page_size % 8 == 0 && (8 * element) % 16 == 0 &&
+  const bool vec = (dim * element) % 16 == 0 && page_size % 8 == 0 &&
                    (static_cast<size_t>(page_size) * element) % 16 == 0 && reinterpret_cast<uintptr_t>(k_pages) % 16 == 0 &&
                    reinterpret_cast<uintptr_t>(v_pages) % 16 == 0;
-#define AKV_ROWS(VEC)                                                                                                   \
+  const unsigned grid = static_cast<unsigned>((rows + kXcds - 1) / kXcds * kXcds);
+#define AKV_ROWS(VEC, G)                                                                                                \
   AKV_DISPATCH(dtype, T,                                                                                                \
-               gated_attention_rows_kernel<T, VEC><<<static_cast<unsigned>((rows + kXcds - 1) / kXcds * kXcds), kRowWaves * kWave, lds, stream>>>(    \
+               gated_attention_rows_kernel<T, VEC, G><<<grid, waves * kWave, lds, stream>>>(                           \
                    static_cast<const T*>(q), static_cast<const T*>(k_pages), static_cast<const T*>(v_pages),            \
                    static_cast<const T*>(gates), gate_stride, gate_at, seq_of_token, positions, block_table, table_rows, \
                    table_width, static_cast<T*>(out), tokens, q_heads, kv_heads, dim, vdim, page_size, num_pages, scale, \
                    softcap, chunk, window, sink, out_stride, out_scale))
-  if (vec) AKV_ROWS(true);
-  else AKV_ROWS(false);
+#define AKV_ROWS_G(VEC)          \
+  switch (bundle) {              \
+    case 4: AKV_ROWS(VEC, 4); break; \
+    case 2: AKV_ROWS(VEC, 2); break; \
+    default: AKV_ROWS(VEC, 1); break; \
+  }
+  if (vec) AKV_ROWS_G(true)
+  else AKV_ROWS_G(false)
+#undef AKV_ROWS_G
 #undef AKV_ROWS
   return AKV_LAUNCH_STATUS();
 }
