@@ -390,10 +390,14 @@ int launch_retention_outputs(const dim3 grid, size_t lds, hipStream_t stream, co
                              int vdim, int rot_dims, const float* table, int table_positions, float key_scale,
                              const float* decay, float eps, const int* q_start, const int* positions, const float* states,
                              int length, int chunks, T* out, long out_stride, float out_scale) {
-  if (lds > 64 * 1024 &&
-      hipFuncSetAttribute(reinterpret_cast<const void*>(&retention_chunk_outputs_kernel<T, GROUPS>),
-                          hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)) != hipSuccess)
-    return -2;
+  // (asked for once per kernel, for the most a launch may want: a step that is being recorded then changes no attribute)
+  static bool allowed = false;
+  if (lds > 64 * 1024 && !allowed) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&retention_chunk_outputs_kernel<T, GROUPS>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024) != hipSuccess)
+      return -2;
+    allowed = true;
+  }
   retention_chunk_outputs_kernel<T, GROUPS><<<grid, 256, lds, stream>>>(projected, stride, heads, dim, vdim, rot_dims, table,
                                                                         table_positions, key_scale, decay, eps, q_start,
                                                                         positions, states, length, chunks, out, out_stride,
@@ -409,10 +413,13 @@ int launch_retention_chunked(const T* projected, long stride, int seqs, int head
                              size_t lds_sums, size_t lds_outputs, hipStream_t stream) {
   const dim3 grid(seqs, heads, chunks);
   const int size = dim * vdim;
-  if (lds_sums > 64 * 1024 &&
-      hipFuncSetAttribute(reinterpret_cast<const void*>(&retention_chunk_sums_kernel<T>),
-                          hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_sums)) != hipSuccess)
-    return -2;
+  static bool allowed = false;
+  if (lds_sums > 64 * 1024 && !allowed) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&retention_chunk_sums_kernel<T>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024) != hipSuccess)
+      return -2;
+    allowed = true;
+  }
   retention_chunk_sums_kernel<T><<<grid, 256, lds_sums, stream>>>(projected, stride, heads, dim, vdim, rot_dims, table,
                                                                 table_positions, key_scale, decay, q_start, positions, sums,
                                                                 length, chunks);

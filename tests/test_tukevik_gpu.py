@@ -75,6 +75,36 @@ def test_steps_are_recorded_and_replayed(case):
     assert torch.equal(outs[True], outs[False])
 
 
+def test_portions_whose_shape_comes_again_are_recorded(tmp_path):
+    """Portions of 32 tokens, again and again, beside a request's single tokens - retention over chunks with a state of
+    128 x 128 (its kernels ask for more than 64 KB of LDS), the matrix-core attention, the scan cut into runs: the
+    recorded steps give the bits of an engine that records nothing, in both arithmetics."""
+    raw = dict(architecture="Tukevik", vocab=200, width=64, norm=dict(eps=1e-6), residual_mult=0.9, layers=[
+        dict(type="parallel", mlp=T.DENSE(64),
+             mixer=T.PARALLEL(T.LEFT(4, 2, 64, 64, 50, 0.8, 10.0), T.RIGHT(1, 128, 128, [0.99], 64, 1e4), 1.0, 1.0)),
+        dict(type="rglru", mixer=T.RGLRU(96, 2, 3), mlp=T.MOE(4, 2, 16, 16))])
+    case = T.make_case("recorded portions", str(tmp_path), (raw, 41, 16))
+    from ampere_kv_engine_amd.engine import StepEntry
+    ids, single = case["requests"]["d"], case["requests"]["b"]
+    for dtype in ("float32", "bfloat16"):
+        outs = {}
+        for graphs in (True, False):
+            engine = T.make_engine(case, dtype, DEVICE, decode_graphs=graphs)
+            d, b = engine.open("d"), engine.open("b")
+            rows = []
+            for step in range(3):          # a step is recorded when its shape comes again; each asks for two rows
+                logits = engine.step([StepEntry(d, ids[32 * step:32 * step + 32], [31]), StepEntry(b, single[step:step + 1], [0])])
+                rows.append(logits.float().cpu())
+            engine.close(d), engine.close(b)
+            got = torch.cat(rows)
+            want = torch.stack([row for step in range(3) for row in (case["expected"]["d"][32 * step + 31], case["expected"]["b"][step])])
+            T.assert_close(got, want, dtype, f"{dtype}, graphs {graphs}")
+            outs[graphs] = got
+            if graphs:
+                assert any(g is not None for g in engine._graphs.values()), "nothing was recorded"
+        assert torch.equal(outs[True], outs[False])
+
+
 def test_trace_replay_of_a_random_model(case, tmp_path):
     """bin/trace_run on a configuration file and a seed: the mixed cutting, every position against the plain model."""
     from ampere_kv_engine_amd.config import TukevikConfig
@@ -167,7 +197,8 @@ def _ctx(lengths_before, counts, device=DEVICE):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("heads,kv_heads,dim,vdim,chunk,page", [(4, 2, 16, 24, 11, 4), (3, 1, 40, 8, 64, 16), (8, 8, 64, 64, 7, 8),
                                                                (2, 1, 128, 256, 300, 16), (8, 2, 64, 32, 20, 16),
-                                                               (4, 4, 32, 128, 48, 32), (1, 1, 64, 64, 5000, 16)])
+                                                               (4, 4, 32, 128, 48, 32), (1, 1, 64, 64, 5000, 16),
+                                                               (2, 1, 256, 32, 40, 16)])
 def test_attention_kernel_alone(hip, dtype, heads, kv_heads, dim, vdim, chunk, page):
     """Two requests in two portions each, through the unit norm with its cache write and the attention, against the plain
     attention of the whole sequences.  Scores are made sharp, and one key a request - the first of a chunk - is made to
