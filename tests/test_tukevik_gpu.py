@@ -133,6 +133,35 @@ def test_trace_replay_of_a_random_model(case, tmp_path):
             row += count
 
 
+def test_the_command_line_generates_with_a_tukevik_model(case, tmp_path):
+    """`python -m ampere_kv_engine_amd.runner` on a configuration file and a seed: one request, and several through the
+    scheduler, greedy; the tokens of the plain implementation.  `--mode check` holds the serving arithmetic against
+    the engine's 32-bit path."""
+    import re
+    from ampere_kv_engine_amd.config import TukevikConfig
+    from ampere_kv_engine_amd.weights import write_random_model
+    config_path = tmp_path / "config.json"
+    config_path.write_text(json.dumps(case["raw"]))
+    folder = write_random_model(str(tmp_path / "model"), TukevikConfig.from_dict(case["raw"]), 5)
+    prompts = [case["requests"]["a"][:19], case["requests"]["b"][:6], case["requests"]["c"][:31]]
+    want = [T.plain_greedy(folder, ids, 6) for ids in prompts]
+    base = [sys.executable, "-m", "ampere_kv_engine_amd.runner", "--random-config", str(config_path), "--weights-seed", "5",
+            "--max-new-tokens", "6", "--ignore-eos"]
+    run = lambda more: subprocess.run(base + more, capture_output=True, text=True, timeout=600, cwd=ROOT)
+    one = run(["--mode", "generate", "--dtype", "float32", "--prompt-ids", " ".join(map(str, prompts[0])), "--prefill-chunk", "8"])
+    assert one.returncode == 0, one.stderr[-2000:]
+    assert json.loads(re.search(r"generated_token_ids = (\[.*\])", one.stdout).group(1)) == want[0]
+    prompts_file = tmp_path / "prompts.txt"
+    prompts_file.write_text("\n".join(" ".join(map(str, ids)) for ids in prompts) + "\n")
+    many = run(["--mode", "generate", "--dtype", "float32", "--prompts-file", str(prompts_file), "--max-seqs", "2",
+                "--prefill-chunk", "5"])
+    assert many.returncode == 0, many.stderr[-2000:]
+    got = [json.loads(line)["generated_token_ids"] for line in many.stdout.splitlines() if line.startswith("{")]
+    assert got == want, many.stdout
+    check = run(["--mode", "check", "--prompt-len", "40"])
+    assert check.returncode == 0, check.stdout[-1500:] + check.stderr[-1500:]
+
+
 def random_configuration(seed: int) -> tuple:
     """Sizes, constants and the order of layers drawn from a seed: any head counts and groupings, keys and values of
     different widths (some no multiple of 8), chunks from one position to longer than a request, any number of blocks
