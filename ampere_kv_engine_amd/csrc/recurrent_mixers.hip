@@ -353,7 +353,8 @@ __global__ __launch_bounds__(1024) void gated_linear_scan_kernel(
         const float r = sigmoid(gates[n * 2 * channels + gate_at] + bias_r);
         const float i = sigmoid(gates[n * 2 * channels + gate_at + block_width] + bias_i);
         a[t] = expf(slope * r);
-        f[t] = sqrtf(1.f - a[t] * a[t]) * i * to_float(u[n * channels + cc]);
+        // 1 - a^2 = -expm1(2 log a): for decays close to 1 the difference of the squares would keep few of its bits
+        f[t] = sqrtf(-expm1f(2.f * slope * r)) * i * to_float(u[n * channels + cc]);
       }
       if (pass == 0) {
 #pragma unroll

@@ -60,7 +60,7 @@ def rglru_scan(u: torch.Tensor, r: torch.Tensor, i: torch.Tensor, lam: torch.Ten
     """S_t = a_t S_(t-1) + sqrt(1 - a_t^2) i_t u_t with a_t = exp(-8 r_t softplus(lam)), from S = 0."""
     log_a = -8.0 * r * softplus(lam)
     a = torch.exp(log_a)
-    gain = torch.sqrt(1.0 - a * a)
+    gain = torch.sqrt(-torch.expm1(2.0 * log_a))         # sqrt(1 - a^2); the difference of squares loses its bits as a nears 1
     state = torch.zeros_like(u[0])
     out = []
     for t in range(u.shape[0]):

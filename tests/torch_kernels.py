@@ -466,7 +466,7 @@ class TorchKernels(KernelSet):
         r = torch.sigmoid(z[..., :bw]).reshape(tokens, width)
         i = torch.sigmoid(z[..., bw:]).reshape(tokens, width)
         a = torch.exp(rate * r)
-        fed = torch.sqrt(1.0 - a * a) * i * u.float()
+        fed = torch.sqrt(-torch.expm1(2.0 * rate * r)) * i * u.float()        # (1 - a^2, without the difference of squares)
         y = xy[:, width:].float()
         y = 0.5 * y * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (y + 0.044715 * y ** 3)))
         for s in range(ctx.num_seqs):
